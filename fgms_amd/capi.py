@@ -1,0 +1,199 @@
+"""ctypes binding of ``include/fgms.h`` (libfgms_hip.so).
+
+The functions take torch GPU tensors only to read their ``data_ptr()`` and
+shapes; nothing torch-specific crosses the C boundary.  There is no CPU
+fallback: if the shared library is missing or a call fails this raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfgms_hip.so")
+
+F32, F16 = 0, 1
+SYMBOLS = [
+    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_destroy",
+    "fgms_plan_usable", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
+    "fgms_wgrad", "fgms_set_kernel_policy",
+]
+
+_lib = None
+
+
+class FgmsError(RuntimeError):
+    pass
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FgmsError("%s is missing: run `python -m fgms_amd.build` (there is no CPU fallback)"
+                        % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.fgms_version.restype = ctypes.c_char_p
+    L.fgms_last_error.restype = ctypes.c_char_p
+    L.fgms_plan_create.argtypes = [ctypes.POINTER(vp), vp, vp, vp, i64, i64, i32, i64, vp]
+    L.fgms_plan_destroy.argtypes = [vp]
+    L.fgms_plan_destroy.restype = None
+    L.fgms_plan_usable.argtypes = [vp, i32]
+    L.fgms_fusion_fwd.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32,
+                                  i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_fwd.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32,
+                           i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_bwd.argtypes = [vp, vp, vp, i32, vp, vp, vp, vp, vp, vp, i32, i32,
+                           i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_dgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_wgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_set_kernel_policy.argtypes = [i32]
+    L.fgms_set_kernel_policy.restype = None
+    _lib = L
+    return L
+
+
+def version():
+    return lib().fgms_version().decode()
+
+
+def _check(rc):
+    if rc != 0:
+        msg = lib().fgms_last_error().decode()
+        if rc == -1:
+            raise ValueError(msg)
+        raise FgmsError("fgms error %d: %s" % (rc, msg))
+
+
+def _dtype(t):
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.float32:
+        return F32
+    raise ValueError("FGMS handles float32 and float16 tensors")
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None and t.numel() else None)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t, name, dtype=None):
+    if not t.is_cuda or not t.is_contiguous():
+        raise ValueError("%s must be a contiguous GPU tensor" % name)
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError("%s must be %s" % (name, dtype))
+
+
+def set_kernel_policy(policy):
+    """0 automatic, 1 generic kernels only, 2 pair-stationary MFMA even with a plan."""
+    lib().fgms_set_kernel_policy(int(policy))
+
+
+class Plan:
+    """Neighbour tables for one kernel map (``fgms_plan_create``)."""
+
+    def __init__(self, kpos, in_map, out_map, n_in, n_out):
+        for t, n in ((kpos, "kpos"), (in_map, "in_map"), (out_map, "out_map")):
+            _need(t, n, torch.int32)
+        self._keep = (kpos, in_map, out_map)
+        self._h = ctypes.c_void_p()
+        _check(lib().fgms_plan_create(ctypes.byref(self._h), _p(kpos), _p(in_map), _p(out_map),
+                                      int(n_in), int(n_out), kpos.numel() - 1, in_map.numel(),
+                                      _stream()))
+
+    @property
+    def handle(self):
+        return self._h
+
+    def usable(self, for_dgrad=False):
+        return bool(lib().fgms_plan_usable(self._h, int(for_dgrad)))
+
+    def close(self):
+        if self._h:
+            lib().fgms_plan_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _ph(plan):
+    return plan.handle if plan is not None else ctypes.c_void_p()
+
+
+def _check_feats(in_feats, kernel):
+    if in_feats.shape[1] != kernel.shape[1]:
+        raise ValueError("Input feature size and kernel size mismatch")
+
+
+def fusion_fwd(in_feats, kernel, sum_nnz, out_feats, kpos, qkpos, in_map, out_map,
+               separate_mid, arch80, plan=None):
+    _check_feats(in_feats, kernel)
+    for t, n in ((in_feats, "in_feats"), (kernel, "kernel"), (out_feats, "out_feats")):
+        _need(t, n, in_feats.dtype)
+    for t, n in ((kpos, "kpos"), (in_map, "in_map"), (out_map, "out_map")):
+        _need(t, n, torch.int32)
+    _check(lib().fgms_fusion_fwd(
+        _p(in_feats), _p(kernel), int(sum_nnz), _p(out_feats), _p(kpos), _p(qkpos), _p(in_map),
+        _p(out_map), int(separate_mid), int(arch80), in_feats.shape[0], out_feats.shape[0],
+        kernel.shape[1], kernel.shape[2], kernel.shape[0], in_map.numel(), _dtype(in_feats),
+        _ph(plan), _stream()))
+
+
+def seq_fwd(in_feats, kernel, sum_nnz, out_feats, kernel_nnz, kernel_pos, in_map, out_map,
+            separate_mid, arch80, plan=None):
+    _check_feats(in_feats, kernel)
+    if kernel_nnz.is_cuda:
+        raise ValueError("kernel_nnz must be a CPU int32 tensor")
+    knnz = kernel_nnz.to(torch.int32).contiguous()
+    for t, n in ((in_feats, "in_feats"), (kernel, "kernel"), (out_feats, "out_feats")):
+        _need(t, n, in_feats.dtype)
+    for t, n in ((kernel_pos, "kernel_pos"), (in_map, "in_map"), (out_map, "out_map")):
+        _need(t, n, torch.int32)
+    _check(lib().fgms_fwd(
+        _p(in_feats), _p(kernel), int(sum_nnz), _p(out_feats), ctypes.c_void_p(knnz.data_ptr()),
+        _p(kernel_pos), _p(in_map), _p(out_map), int(separate_mid), int(arch80),
+        in_feats.shape[0], out_feats.shape[0], kernel.shape[1], kernel.shape[2], kernel.shape[0],
+        in_map.numel(), _dtype(in_feats), _ph(plan), _stream()))
+
+
+def bwd(out_grad, in_feats, kernel, sum_nnz, in_grad, kernel_grad, kpos, qkpos, in_map,
+        out_map, separate_mid, arch80, plan=None):
+    _check_feats(in_feats, kernel)
+    for t, n in ((out_grad, "out_feats_grad"), (in_feats, "in_feats"), (kernel, "kernel"),
+                 (in_grad, "in_feats_grad"), (kernel_grad, "kernel_grad")):
+        _need(t, n, in_feats.dtype)
+    for t, n in ((kpos, "kpos"), (in_map, "in_map"), (out_map, "out_map")):
+        _need(t, n, torch.int32)
+    _check(lib().fgms_bwd(
+        _p(out_grad), _p(in_feats), _p(kernel), int(sum_nnz), _p(in_grad), _p(kernel_grad),
+        _p(kpos), _p(qkpos), _p(in_map), _p(out_map), int(separate_mid), int(arch80),
+        in_feats.shape[0], out_grad.shape[0], kernel.shape[1], kernel.shape[2], kernel.shape[0],
+        in_map.numel(), _dtype(in_feats), _ph(plan), _stream()))
+
+
+def dgrad(out_grad, kernel, in_grad, kpos, in_map, out_map, plan=None):
+    for t, n in ((out_grad, "out_feats_grad"), (kernel, "kernel"), (in_grad, "in_feats_grad")):
+        _need(t, n, out_grad.dtype)
+    _check(lib().fgms_dgrad(
+        _p(out_grad), _p(kernel), _p(in_grad), _p(kpos), _p(in_map), _p(out_map),
+        in_grad.shape[0], out_grad.shape[0], kernel.shape[1], kernel.shape[2], kernel.shape[0],
+        in_map.numel(), _dtype(out_grad), _ph(plan), _stream()))
+
+
+def wgrad(in_feats, out_grad, kernel_grad, kpos, in_map, out_map, plan=None):
+    for t, n in ((in_feats, "in_feats"), (out_grad, "out_feats_grad"), (kernel_grad, "kernel_grad")):
+        _need(t, n, in_feats.dtype)
+    _check(lib().fgms_wgrad(
+        _p(in_feats), _p(out_grad), _p(kernel_grad), _p(kpos), _p(in_map), _p(out_map),
+        in_feats.shape[0], out_grad.shape[0], kernel_grad.shape[1], kernel_grad.shape[2],
+        kernel_grad.shape[0], in_map.numel(), _dtype(in_feats), _ph(plan), _stream()))

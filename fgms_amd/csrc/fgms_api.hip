@@ -1,0 +1,257 @@
+// extern "C" entry points of libfgms_hip.so: argument checks, kernel selection,
+// workspace bookkeeping.  The host-side counterpart of backend/spconv.cu:23-571.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <map>
+#include <mutex>
+#include <utility>
+
+#include "fgms_internal.h"
+
+namespace fgms {
+
+static thread_local char g_error[512] = "";
+static int g_policy = 0;
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+// ---- workspace: one growable buffer per (device, stream, slot) --------------
+namespace {
+struct WsKey {
+  int device;
+  hipStream_t stream;
+  int slot;
+  bool operator<(const WsKey &o) const {
+    if (device != o.device) return device < o.device;
+    if (stream != o.stream) return stream < o.stream;
+    return slot < o.slot;
+  }
+};
+struct WsBuf {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_ws_mutex;
+std::map<WsKey, WsBuf> g_ws;
+}  // namespace
+
+int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr) {
+  int dev = 0;
+  FGMS_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  WsBuf &b = g_ws[WsKey{dev, stream, slot}];
+  if (b.bytes < bytes) {
+    if (b.ptr) {
+      // the old buffer may still be in use by work queued on this stream
+      FGMS_HIP_TRY(hipStreamSynchronize(stream));
+      FGMS_HIP_TRY(hipFree(b.ptr));
+      b.ptr = nullptr;
+      b.bytes = 0;
+    }
+    size_t want = bytes + bytes / 4 + 4096;
+    if (hipMalloc(&b.ptr, want) != hipSuccess) {
+      b.ptr = nullptr;
+      set_error("workspace allocation of %zu bytes failed", want);
+      return FGMS_E_NOMEM;
+    }
+    b.bytes = want;
+  }
+  *ptr = b.ptr;
+  return FGMS_OK;
+}
+
+namespace {
+
+int check_common(const void *a, const void *b, const void *c, const int32_t *kpos,
+                 const int32_t *imap, const int32_t *omap, int64_t n_in, int64_t n_out, int c_in,
+                 int c_out, int k_vol, int64_t n_pairs, int dtype) {
+  if (dtype != FGMS_F32 && dtype != FGMS_F16) {
+    set_error("dtype must be FGMS_F32 (0) or FGMS_F16 (1), got %d", dtype);
+    return FGMS_E_INVALID;
+  }
+  if (n_in < 0 || n_out < 0 || c_in <= 0 || c_out <= 0 || k_vol <= 0 || n_pairs < 0) {
+    set_error("bad sizes: n_in=%lld n_out=%lld c_in=%d c_out=%d k_vol=%d n_pairs=%lld",
+              (long long)n_in, (long long)n_out, c_in, c_out, k_vol, (long long)n_pairs);
+    return FGMS_E_INVALID;
+  }
+  if (n_in > INT32_MAX || n_out > INT32_MAX || n_pairs > INT32_MAX - 65536) {
+    set_error("row and pair counts must fit int32 (the maps are int32)");
+    return FGMS_E_INVALID;
+  }
+  if (!kpos || (n_pairs > 0 && (!imap || !omap)) ||
+      ((n_in > 0 || n_out > 0) && (!a || !b || !c))) {
+    set_error("null pointer argument");
+    return FGMS_E_INVALID;
+  }
+  return FGMS_OK;
+}
+
+int run_gms(GmsArgs a, const Plan *plan) {
+  const bool dense = a.dense_k >= 0;
+  if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
+  if (g_policy != 1) {
+    if (!dense && g_policy != 2 && planned_gms_supported(a, plan)) return launch_planned_gms(a, plan);
+    if (mfma_gms_supported(a)) return launch_mfma_gms(a);
+  }
+  return launch_generic_gms(a);
+}
+
+int run_wgrad(const WgradArgs &a) {
+  if (a.n_pairs == 0) return FGMS_OK;
+  if (g_policy != 1 && mfma_wgrad_supported(a)) return launch_mfma_wgrad(a);
+  return launch_generic_wgrad(a);
+}
+
+int mid_of(int k_vol) { return (k_vol % 2 == 1) ? k_vol / 2 : 0; }
+
+GmsArgs fwd_args(const void *in, const void *w, void *out, const int32_t *kpos,
+                 const int32_t *imap, const int32_t *omap, int64_t n_in, int64_t n_out, int c_in,
+                 int c_out, int k_vol, int64_t n_pairs, int dtype, hipStream_t s) {
+  GmsArgs a{};
+  a.src = in; a.w = w; a.dst = out; a.kpos = kpos; a.gmap = imap; a.smap = omap;
+  a.n_src = n_in; a.n_dst = n_out; a.c_in = c_in; a.c_out = c_out; a.k_vol = k_vol;
+  a.n_pairs = n_pairs; a.transpose_w = false; a.dense_k = -1; a.n_dense = 0; a.dtype = dtype;
+  a.stream = s;
+  return a;
+}
+
+int check_mid(int separate_mid, int64_t n_in, int64_t n_out) {
+  if (separate_mid && n_in != n_out) {
+    set_error("separate_mid needs n_in == n_out (got %lld, %lld)", (long long)n_in, (long long)n_out);
+    return FGMS_E_INVALID;
+  }
+  return FGMS_OK;
+}
+
+}  // namespace
+}  // namespace fgms
+
+using namespace fgms;
+
+extern "C" {
+
+const char *fgms_version(void) { return "fgms-hip 0.1 (gfx950)"; }
+const char *fgms_last_error(void) { return g_error; }
+void fgms_set_kernel_policy(int policy) { g_policy = policy; }
+
+int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_feats,
+                    const int32_t *kpos, const int32_t *qkpos, const int32_t *in_map,
+                    const int32_t *out_map, int separate_mid, int arch80, int64_t n_in,
+                    int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype,
+                    fgms_plan_t *plan, void *stream) {
+  (void)sum_nnz; (void)qkpos; (void)arch80;
+  int rc = check_common(in_feats, kernel, out_feats, kpos, in_map, out_map, n_in, n_out, c_in,
+                        c_out, k_vol, n_pairs, dtype);
+  if (rc) return rc;
+  if ((rc = check_mid(separate_mid, n_in, n_out))) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  GmsArgs a = fwd_args(in_feats, kernel, out_feats, kpos, in_map, out_map, n_in, n_out, c_in,
+                       c_out, k_vol, n_pairs, dtype, s);
+  if (separate_mid) {
+    // centre product first and overwriting, as the beta = 0 GEMM of the reference
+    const size_t esz = dtype == FGMS_F16 ? 2 : 4;
+    if ((rc = launch_fill_zero(out_feats, (size_t)n_out * c_out * esz, s))) return rc;
+    GmsArgs d = a;
+    d.gmap = d.smap = nullptr;
+    d.dense_k = mid_of(k_vol);
+    d.n_dense = n_out;
+    if ((rc = run_gms(d, nullptr))) return rc;
+  }
+  return run_gms(a, (const Plan *)plan);
+}
+
+int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_feats,
+             const int32_t *kernel_nnz, const int32_t *kernel_pos, const int32_t *in_map,
+             const int32_t *out_map, int separate_mid, int arch80, int64_t n_in, int64_t n_out,
+             int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype, fgms_plan_t *plan,
+             void *stream) {
+  (void)sum_nnz; (void)arch80;
+  int rc = check_common(in_feats, kernel, out_feats, kernel_pos, in_map, out_map, n_in, n_out,
+                        c_in, c_out, k_vol, n_pairs, dtype);
+  if (rc) return rc;
+  if ((rc = check_mid(separate_mid, n_in, n_out))) return rc;
+  if (!kernel_nnz) {
+    set_error("kernel_nnz (host int32[k_vol]) is null");
+    return FGMS_E_INVALID;
+  }
+  // The host-side counts bound the pair range exactly (the reference walks them
+  // to slice the maps, backend/spconv.cu:307-324).
+  int64_t total = 0;
+  for (int k = 0; k < k_vol; ++k) {
+    if (kernel_nnz[k] < 0) {
+      set_error("kernel_nnz[%d] is negative", k);
+      return FGMS_E_INVALID;
+    }
+    total += kernel_nnz[k];
+  }
+  if (total > n_pairs) {
+    set_error("kernel_nnz sums to %lld but the maps hold %lld pairs", (long long)total,
+              (long long)n_pairs);
+    return FGMS_E_INVALID;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  GmsArgs a = fwd_args(in_feats, kernel, out_feats, kernel_pos, in_map, out_map, n_in, n_out,
+                       c_in, c_out, k_vol, total, dtype, s);
+  if ((rc = run_gms(a, (const Plan *)plan))) return rc;
+  if (separate_mid) {
+    GmsArgs d = a;
+    d.gmap = d.smap = nullptr;
+    d.dense_k = mid_of(k_vol);
+    d.n_dense = n_out;
+    if ((rc = run_gms(d, nullptr))) return rc;
+  }
+  return FGMS_OK;
+}
+
+int fgms_dgrad(const void *out_feats_grad, const void *kernel, void *in_feats_grad,
+               const int32_t *kpos, const int32_t *in_map, const int32_t *out_map, int64_t n_in,
+               int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype,
+               fgms_plan_t *plan, void *stream) {
+  int rc = check_common(out_feats_grad, kernel, in_feats_grad, kpos, in_map, out_map, n_in, n_out,
+                        c_in, c_out, k_vol, n_pairs, dtype);
+  if (rc) return rc;
+  GmsArgs a{};
+  a.src = out_feats_grad; a.w = kernel; a.dst = in_feats_grad; a.kpos = kpos;
+  a.gmap = out_map; a.smap = in_map;   // roles swap, as at backend/spconv.cu:460,559
+  a.n_src = n_out; a.n_dst = n_in; a.c_in = c_in; a.c_out = c_out; a.k_vol = k_vol;
+  a.n_pairs = n_pairs; a.transpose_w = true; a.dense_k = -1; a.n_dense = 0; a.dtype = dtype;
+  a.stream = (hipStream_t)stream;
+  return run_gms(a, (const Plan *)plan);
+}
+
+int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_grad,
+               const int32_t *kpos, const int32_t *in_map, const int32_t *out_map, int64_t n_in,
+               int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype,
+               fgms_plan_t *plan, void *stream) {
+  (void)plan;
+  int rc = check_common(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
+                        c_in, c_out, k_vol, n_pairs, dtype);
+  if (rc) return rc;
+  WgradArgs a{};
+  a.in = in_feats; a.gout = out_feats_grad; a.gw = kernel_grad; a.kpos = kpos;
+  a.imap = in_map; a.omap = out_map; a.n_in = n_in; a.n_out = n_out; a.c_in = c_in;
+  a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
+  a.stream = (hipStream_t)stream;
+  return run_wgrad(a);
+}
+
+int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kernel, int sum_nnz,
+             void *in_feats_grad, void *kernel_grad, const int32_t *kpos, const int32_t *qkpos,
+             const int32_t *in_map, const int32_t *out_map, int separate_mid, int arch80,
+             int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs,
+             int dtype, fgms_plan_t *plan, void *stream) {
+  (void)sum_nnz; (void)qkpos; (void)separate_mid; (void)arch80;
+  int rc = fgms_dgrad(out_feats_grad, kernel, in_feats_grad, kpos, in_map, out_map, n_in, n_out,
+                      c_in, c_out, k_vol, n_pairs, dtype, plan, stream);
+  if (rc) return rc;
+  return fgms_wgrad(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
+                    c_in, c_out, k_vol, n_pairs, dtype, plan, stream);
+}
+
+}  // extern "C"

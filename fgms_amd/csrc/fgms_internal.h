@@ -1,0 +1,90 @@
+// Internal declarations shared by the translation units of libfgms_hip.so.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fgms.h"
+
+namespace fgms {
+
+void set_error(const char *fmt, ...);
+
+#define FGMS_HIP_TRY(expr)                                                     \
+  do {                                                                         \
+    hipError_t e_ = (expr);                                                    \
+    if (e_ != hipSuccess) {                                                    \
+      ::fgms::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                        __FILE__, __LINE__);                                   \
+      return FGMS_E_HIP;                                                       \
+    }                                                                          \
+  } while (0)
+
+// One gather-GEMM-scatter pass over a pair list.
+//   dst[smap[j], :] += src[gmap[j], :] @ op(W[k])      for j in [kpos[k], kpos[k+1])
+// forward: src = in_feats, dst = out_feats, gmap = in_map, smap = out_map,
+//          op(W) = W            (c_src = c_in,  c_dst = c_out)
+// dgrad:   src = out_grad, dst = in_grad, gmap = out_map, smap = in_map,
+//          op(W) = W^T          (c_src = c_out, c_dst = c_in)
+// dense:   gmap == smap == nullptr means the identity map over n_dense rows of
+//          the single offset `dense_k` (the separately handled centre offset).
+struct GmsArgs {
+  const void *src;
+  const void *w;      // [k_vol, c_in, c_out]
+  void *dst;
+  const int32_t *kpos;
+  const int32_t *gmap;
+  const int32_t *smap;
+  int64_t n_src, n_dst;
+  int c_in, c_out;    // the weight's own shape, whatever the direction
+  int k_vol;
+  int64_t n_pairs;    // upper bound on kpos[k_vol]
+  bool transpose_w;   // dgrad
+  int dense_k;        // >= 0: identity map over n_dense rows with W[dense_k]
+  int64_t n_dense;
+  int dtype;
+  hipStream_t stream;
+};
+
+struct WgradArgs {
+  const void *in;     // [n_in, c_in]
+  const void *gout;   // [n_out, c_out]
+  void *gw;           // [k_vol, c_in, c_out]
+  const int32_t *kpos;
+  const int32_t *imap;
+  const int32_t *omap;
+  int64_t n_in, n_out;
+  int c_in, c_out, k_vol;
+  int64_t n_pairs;
+  int dtype;
+  hipStream_t stream;
+};
+
+// Plan: neighbour tables built from the pair lists.
+struct Plan {
+  int device;
+  int k_vol;
+  int64_t n_in, n_out, n_pairs;
+  int32_t *nbr_out;   // [n_out, k_vol]: input row feeding output row o through offset k, or -1
+  int32_t *nbr_in;    // [n_in,  k_vol]: output row fed by input row i through offset k, or -1
+  bool fwd_ok;        // no offset maps two pairs onto one output row
+  bool dgrad_ok;      // no offset maps two pairs from one input row
+};
+
+// Fp32 scratch that outlives a call (per device and stream, grown on demand).
+// slot 0: packed weights, slot 1: fp32 weight-gradient accumulator.
+int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr);
+
+// ---- launchers (each returns an FGMS_* code) ----
+int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+int launch_generic_gms(const GmsArgs &a);
+int launch_generic_wgrad(const WgradArgs &a);
+bool mfma_gms_supported(const GmsArgs &a);
+int launch_mfma_gms(const GmsArgs &a);
+bool mfma_wgrad_supported(const WgradArgs &a);
+int launch_mfma_wgrad(const WgradArgs &a);
+bool planned_gms_supported(const GmsArgs &a, const Plan *p);
+int launch_planned_gms(const GmsArgs &a, const Plan *p);
+
+}  // namespace fgms

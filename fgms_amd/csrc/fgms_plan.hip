@@ -1,0 +1,137 @@
+// Kernel-map plan: neighbour tables built on the device from the pair lists.
+// nbr_out[o][k] = the input row that reaches output row o through offset k
+// (-1 if none); nbr_in[i][k] = the output row that input row i reaches through
+// offset k.  The reference keeps only the pair lists and scatters with atomics
+// (backend/spconv.cuh:457-563); the tables let a workgroup own a block of
+// output rows and sum all offsets in registers.
+#include "fgms_device.h"
+#include "fgms_internal.h"
+
+namespace fgms {
+namespace {
+
+__global__ void fill_i32_kernel(int32_t *__restrict__ p, size_t n, int32_t v) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = v;
+}
+
+// flags[0]: an index is out of range; flags[1]: two pairs of one offset share
+// an output row; flags[2]: two pairs of one offset share an input row.
+__global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
+                                    const int32_t *__restrict__ imap,
+                                    const int32_t *__restrict__ omap, int k_vol, int n_in,
+                                    int n_out, int32_t *__restrict__ nbr_out,
+                                    int32_t *__restrict__ nbr_in, int *__restrict__ flags) {
+  const int total = kpos[k_vol];
+  int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= total) return;
+  // offset of pair j: the last k with kpos[k] <= j
+  int lo = 0, hi = k_vol;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (kpos[mid] <= j) lo = mid; else hi = mid;
+  }
+  const int k = lo;
+  const int i = imap[j], o = omap[j];
+  if (i < 0 || i >= n_in || o < 0 || o >= n_out) {
+    flags[0] = 1;
+    return;
+  }
+  if (atomicCAS(&nbr_out[(size_t)o * k_vol + k], -1, i) != -1) flags[1] = 1;
+  if (atomicCAS(&nbr_in[(size_t)i * k_vol + k], -1, o) != -1) flags[2] = 1;
+}
+
+int fill_i32(int32_t *p, size_t n, int32_t v, hipStream_t s) {
+  if (n == 0) return FGMS_OK;
+  size_t blocks = (n + 1023) / 1024;
+  if (blocks > 65535) blocks = 65535;
+  fill_i32_kernel<<<(unsigned)blocks, 256, 0, s>>>(p, n, v);
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
+}  // namespace
+}  // namespace fgms
+
+using namespace fgms;
+
+extern "C" {
+
+int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
+                     const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
+                     int64_t n_pairs, void *stream) {
+  if (!plan_out) {
+    set_error("plan output pointer is null");
+    return FGMS_E_INVALID;
+  }
+  *plan_out = nullptr;
+  if (!kpos || k_vol <= 0 || n_in < 0 || n_out < 0 || n_pairs < 0 ||
+      (n_pairs > 0 && (!in_map || !out_map)) || n_in > INT32_MAX || n_out > INT32_MAX ||
+      n_pairs > INT32_MAX - 65536) {
+    set_error("fgms_plan_create: bad argument");
+    return FGMS_E_INVALID;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  Plan *p = new Plan();
+  p->k_vol = k_vol; p->n_in = n_in; p->n_out = n_out; p->n_pairs = n_pairs;
+  p->nbr_out = p->nbr_in = nullptr; p->fwd_ok = p->dgrad_ok = false;
+  int *flags = nullptr;
+  int rc = FGMS_OK;
+  auto fail = [&](int code) {
+    if (flags) (void)hipFree(flags);
+    fgms_plan_destroy((fgms_plan_t *)p);
+    return code;
+  };
+  if (hipGetDevice(&p->device) != hipSuccess) return fail(FGMS_E_HIP);
+  const size_t so = (size_t)n_out * k_vol, si = (size_t)n_in * k_vol;
+  if (hipMalloc((void **)&p->nbr_out, (so ? so : 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc((void **)&p->nbr_in, (si ? si : 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc((void **)&flags, 4 * sizeof(int)) != hipSuccess) {
+    set_error("fgms_plan_create: table allocation failed");
+    return fail(FGMS_E_NOMEM);
+  }
+  if ((rc = fill_i32(p->nbr_out, so, -1, s))) return fail(rc);
+  if ((rc = fill_i32(p->nbr_in, si, -1, s))) return fail(rc);
+  if ((rc = fill_i32(flags, 4, 0, s))) return fail(rc);
+  if (n_pairs > 0) {
+    build_tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
+        kpos, in_map, out_map, k_vol, (int)n_in, (int)n_out, p->nbr_out, p->nbr_in, flags);
+    if (hipGetLastError() != hipSuccess) {
+      set_error("fgms_plan_create: table build launch failed");
+      return fail(FGMS_E_HIP);
+    }
+  }
+  int h[4] = {0, 0, 0, 0};
+  if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
+      hipStreamSynchronize(s) != hipSuccess) {
+    set_error("fgms_plan_create: reading the build flags failed");
+    return fail(FGMS_E_HIP);
+  }
+  (void)hipFree(flags);
+  flags = nullptr;
+  if (h[0]) {
+    set_error("fgms_plan_create: a map index is outside [0, n_in) x [0, n_out)");
+    return fail(FGMS_E_INVALID);
+  }
+  p->fwd_ok = !h[1];
+  p->dgrad_ok = !h[2];
+  *plan_out = (fgms_plan_t *)p;
+  return FGMS_OK;
+}
+
+void fgms_plan_destroy(fgms_plan_t *plan) {
+  Plan *p = (Plan *)plan;
+  if (!p) return;
+  if (p->nbr_out) (void)hipFree(p->nbr_out);
+  if (p->nbr_in) (void)hipFree(p->nbr_in);
+  delete p;
+}
+
+int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad) {
+  const Plan *p = (const Plan *)plan;
+  if (!p) return 0;
+  return for_dgrad ? (p->dgrad_ok ? 1 : 0) : (p->fwd_ok ? 1 : 0);
+}
+
+}  // extern "C"

@@ -1,0 +1,139 @@
+/*
+ * fgms.h -- C ABI of the MI355X (gfx950) fused gather-GEMM-scatter library.
+ *
+ * One entry point per function that hkeee21/FGMS exports through pybind
+ * (backend/pybind_cuda.cpp:8-10, declared in backend/spconv.h:10-49).  Tensors
+ * become raw device pointers plus the sizes the reference reads off the
+ * at::Tensor arguments (backend/spconv.cu:36-48); everything else keeps the
+ * reference's name, order and meaning.
+ *
+ * Conventions shared by all entry points
+ *   - in_feats  [n_in,  c_in ]  row-major, device
+ *   - kernel    [k_vol, c_in, c_out] row-major, device
+ *   - out_feats [n_out, c_out]  row-major, device, caller-zeroed, accumulated
+ *   - in_map / out_map: int32[n_pairs], device; the pairs of offset k occupy
+ *     [kpos[k], kpos[k+1]); pair j adds in_feats[in_map[j]] @ kernel[k] to
+ *     out_feats[out_map[j]].
+ *   - kpos: int32[k_vol+1] device, exclusive prefix sum of the per-offset pair
+ *     counts.  qkpos / sum_nnz (the 256-padded prefix sum and its total,
+ *     cpu-check.py:6-14) are accepted for signature compatibility; tile
+ *     scheduling is derived from kpos, so any padding quantum works.
+ *   - dtype: FGMS_F32 or FGMS_F16 for features, weights and gradients alike
+ *     (the reference keys on in_feats.scalar_type(), backend/spconv.cu:47-48).
+ *   - arch80: for FGMS_F32, non-zero = "tf32 mode" in the reference
+ *     (backend/spconv.cu:67-68,213).  gfx950 has no xf32 MFMA: both modes run
+ *     the fp32 MFMA kernels, so tf32 mode is simply more exact than asked.
+ *   - stream: a hipStream_t (NULL = the null stream).  All work is enqueued on
+ *     it; calls return without waiting for the GPU, as the reference's do.
+ *   - plan: optional (NULL allowed) handle from fgms_plan_create for the same
+ *     maps; with a plan the output-stationary kernels run (no atomics,
+ *     deterministic), without one the pair-stationary atomic kernels run.
+ *   - return value: 0 on success, a negative FGMS_E_* code otherwise;
+ *     fgms_last_error() describes the last failure on the calling thread.
+ */
+#ifndef FGMS_H_
+#define FGMS_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGMS_F32 0
+#define FGMS_F16 1
+
+#define FGMS_OK 0
+#define FGMS_E_INVALID (-1)   /* bad argument (shape, dtype, null pointer)   */
+#define FGMS_E_HIP (-2)       /* a HIP runtime call failed                    */
+#define FGMS_E_NOMEM (-3)     /* workspace / plan allocation failed           */
+
+typedef struct fgms_plan fgms_plan_t;
+
+/* Library identification; also proves the shared object loads. */
+const char *fgms_version(void);
+const char *fgms_last_error(void);
+
+/*
+ * Kernel-map plan.  Built once per (in_map, out_map, kpos) on the device and
+ * reusable by every layer and every pass that shares the map: a neighbour
+ * table "output row x offset -> input row" (and its transpose for dgrad).  The
+ * reference has no counterpart: it re-reads the pair lists on every call
+ * (backend/spconv.cuh:457-563).  Creation synchronises `stream` once to learn
+ * whether some offset maps two pairs onto one output row (then the plan is
+ * marked non-functional and the entry points silently use the atomic kernels).
+ */
+int fgms_plan_create(fgms_plan_t **plan, const int32_t *kpos,
+                     const int32_t *in_map, const int32_t *out_map,
+                     int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
+                     void *stream);
+void fgms_plan_destroy(fgms_plan_t *plan);
+/* 1 if the output-stationary kernels can use it for forward / for dgrad. */
+int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad);
+
+/*
+ * Replaces ConvolutionForwardFused  (backend/spconv.cu:23-246; pybind name
+ * fgms_fusion_fwd_cuda, backend/pybind_cuda.cpp:8).
+ * separate_mid != 0: the centre offset (k_vol/2 for odd k_vol, else 0,
+ * backend/spconv.cu:52) is not in the map; out_feats is first OVERWRITTEN with
+ * in_feats @ kernel[mid] (GEMM with beta = 0, backend/spconv.cu:56,76-106), so
+ * n_in must equal n_out, and the map's pairs are accumulated on top.
+ */
+int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz,
+                    void *out_feats, const int32_t *kpos, const int32_t *qkpos,
+                    const int32_t *in_map, const int32_t *out_map,
+                    int separate_mid, int arch80,
+                    int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
+                    int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
+
+/*
+ * Replaces ConvolutionForward  (backend/spconv.cu:249-411; pybind name
+ * fgms_fwd_cuda, backend/pybind_cuda.cpp:9): the per-offset "sequential" form.
+ * kernel_nnz is a HOST array int32[k_vol] (backend/spconv.cu:308); kernel_pos
+ * is the device kpos.  With separate_mid the centre product is ADDED after the
+ * map's pairs (beta = 1, backend/spconv.cu:377-410).
+ */
+int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz,
+             void *out_feats, const int32_t *kernel_nnz, const int32_t *kernel_pos,
+             const int32_t *in_map, const int32_t *out_map,
+             int separate_mid, int arch80,
+             int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
+             int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
+
+/*
+ * Replaces ConvolutionBackward  (backend/spconv.cu:414-571; pybind name
+ * fgms_bwd_cuda, backend/pybind_cuda.cpp:10): input gradient, then weight
+ * gradient, both accumulated into caller-zeroed buffers.  separate_mid and
+ * arch80 are accepted and ignored, as in the reference.
+ *   in_feats_grad[in_map[j]]  += out_feats_grad[out_map[j]] @ kernel[k]^T
+ *   kernel_grad[k]            += in_feats[in_map[j]]^T (x) out_feats_grad[out_map[j]]
+ */
+int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kernel,
+             int sum_nnz, void *in_feats_grad, void *kernel_grad,
+             const int32_t *kpos, const int32_t *qkpos,
+             const int32_t *in_map, const int32_t *out_map,
+             int separate_mid, int arch80,
+             int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
+             int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
+
+/* The two halves of fgms_bwd on their own (the reference launches them back to
+ * back, backend/spconv.cu:454-461 + 495-548 / 553-569); exposed so each can be
+ * timed and tested separately. */
+int fgms_dgrad(const void *out_feats_grad, const void *kernel, void *in_feats_grad,
+               const int32_t *kpos, const int32_t *in_map, const int32_t *out_map,
+               int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
+               int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
+int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_grad,
+               const int32_t *kpos, const int32_t *in_map, const int32_t *out_map,
+               int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
+               int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
+
+/* Selects kernels by hand for tests and profiling: 0 = automatic dispatch,
+ * 1 = force the generic (non-MFMA) kernels, 2 = force the pair-stationary MFMA
+ * kernels even when a usable plan is passed.  Process-wide. */
+void fgms_set_kernel_policy(int policy);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FGMS_H_ */

@@ -1,0 +1,215 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle
+on identical seeded inputs.  Tolerances: fp32 rel 1e-5, tf32 / fp16 rel 1e-2
+(see gpu_util.assert_close); index handling bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from fgms_amd import clouds
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from fgms_amd import capi as c
+    c.lib()
+    assert torch.cuda.is_available()
+    yield c
+    c.set_kernel_policy(0)
+
+
+def cloud(seed, n=3000, grid=24):
+    rng = np.random.default_rng(seed)
+    pts = np.concatenate([
+        clouds._patch(rng, rng.uniform(6, 18, 3), 9, 9, oblique=False),
+        clouds._patch(rng, rng.uniform(6, 18, 3), 9, 9, oblique=True),
+        clouds._sphere_shell(rng, np.array([12., 12, 12]), 7.0, n),
+    ])
+    return clouds.dedup(pts, grid)
+
+
+def layer(seed, c_in, c_out, dtype, kind="subm"):
+    rng = np.random.default_rng(seed)
+    vox = cloud(seed)
+    if kind == "subm":
+        return clouds.submanifold_case(vox, c_in, c_out, dtype, rng)
+    coarse = clouds.downsample_coords(vox, 2)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vox, coarse, clouds.offsets_cube(2), 2)
+    if kind == "down":
+        return clouds.make_layer(rng, imap, omap, knnz, kpos, len(vox), len(coarse), c_in, c_out, dtype)
+    return clouds.make_layer(rng, omap, imap, knnz, kpos, len(coarse), len(vox), c_in, c_out, dtype)
+
+
+def check_all(capi, oracle, L, policy, use_plan, arch80=False):
+    capi.set_kernel_policy(policy)
+    D = G.to_dev(L)
+    mode = G.mode_of(L["in_feats"].dtype, arch80)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"]) if use_plan else None
+    args = (L["knnz"], L["imap"], L["omap"])
+    ref = oracle.np_fwd(L["in_feats"], L["kernel"], *args, L["n_out"])
+    G.assert_close(G.run_fwd(capi, D, fused=True, arch80=arch80, plan=plan), ref, mode, "fused fwd")
+    G.assert_close(G.run_fwd(capi, D, fused=False, arch80=arch80, plan=plan), ref, mode, "seq fwd")
+    gi, gw = G.run_bwd(capi, D, plan=plan)
+    bmode = mode if mode != "fp32" else "fp32"
+    G.assert_close(gi, oracle.np_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"]), bmode, "dgrad")
+    G.assert_close(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"]), bmode, "wgrad")
+    if plan is not None:
+        plan.close()
+
+
+SHAPES = [(32, 32), (64, 64), (16, 16), (4, 32), (3, 5), (128, 128), (64, 128), (128, 64), (48, 80), (8, 8)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "%dx%d" % s)
+def test_submanifold_auto(capi, oracle, shape, dtype):
+    L = layer(11, shape[0], shape[1], dtype)
+    check_all(capi, oracle, L, policy=0, use_plan=False)
+    check_all(capi, oracle, L, policy=0, use_plan=True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("shape", [(32, 32), (64, 64), (3, 5), (128, 64)], ids=lambda s: "%dx%d" % s)
+def test_submanifold_generic_kernels(capi, oracle, shape, dtype):
+    check_all(capi, oracle, layer(12, shape[0], shape[1], dtype), policy=1, use_plan=False)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("shape", [(32, 32), (64, 64), (128, 128), (64, 128)], ids=lambda s: "%dx%d" % s)
+def test_submanifold_pair_stationary_mfma(capi, oracle, shape, dtype):
+    check_all(capi, oracle, layer(13, shape[0], shape[1], dtype), policy=2, use_plan=True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("kind,shape", [("down", (64, 128)), ("up", (128, 64)), ("down", (16, 32)), ("up", (5, 3))])
+def test_strided_and_transposed(capi, oracle, kind, shape, dtype):
+    L = layer(14, shape[0], shape[1], dtype, kind)
+    check_all(capi, oracle, L, policy=0, use_plan=False)
+    check_all(capi, oracle, L, policy=0, use_plan=True)
+
+
+def test_tf32_mode_flag(capi, oracle):
+    check_all(capi, oracle, layer(15, 64, 64, np.float32), policy=0, use_plan=True, arch80=True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "seq"])
+def test_separate_mid(capi, oracle, fused, dtype):
+    """Centre offset left out of the map (knnz[13] == 0) and added as a dense
+    product, the form the reference's tiny samples take (cpu-check.py:100)."""
+    rng = np.random.default_rng(16)
+    vox = cloud(16)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vox, vox, clouds.offsets_cube(3), skip_offset=13)
+    L = clouds.make_layer(rng, imap, omap, knnz, kpos, len(vox), len(vox), 32, 64, dtype)
+    D = G.to_dev(L)
+    ref = oracle.np_fwd(L["in_feats"], L["kernel"], knnz, imap, omap, len(vox), precompute=True)
+    mode = G.mode_of(dtype)
+    for use_plan in (False, True):
+        plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"]) if use_plan else None
+        G.assert_close(G.run_fwd(capi, D, fused=fused, separate_mid=True, plan=plan), ref, mode)
+    if fused:
+        # the fused form overwrites (GEMM beta = 0, backend/spconv.cu:56): junk in out must vanish
+        junk = torch.full((len(vox), 64), 7.0, dtype=D["in_feats"].dtype, device="cuda")
+        G.assert_close(G.run_fwd(capi, D, fused=True, separate_mid=True, out_init=junk), ref, mode)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+def test_accumulates_in_place(capi, oracle, dtype):
+    L = layer(17, 32, 32, dtype)
+    D = G.to_dev(L)
+    base = torch.randn(D["n_out"], 32, device="cuda").to(D["in_feats"].dtype)
+    ref = base.float().cpu().numpy().astype(np.float64) + oracle.np_fwd(
+        L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
+    for use_plan in (False, True):
+        plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"]) if use_plan else None
+        G.assert_close(G.run_fwd(capi, D, plan=plan, out_init=base), ref, G.mode_of(dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+def test_index_handling_bit_exact(capi, dtype):
+    """W[k] = identity and every output row hit by exactly one pair: the result
+    is a permutation copy, so any index slip shows as a bit difference."""
+    rng = np.random.default_rng(18)
+    n_in, n_out, c, k_vol = 5000, 4000, 64, 8
+    knnz = np.array([0, 700, 1, 0, 2000, 255, 257, 787], np.int32)
+    kpos = np.concatenate([[0], np.cumsum(knnz)]).astype(np.int32)
+    omap = rng.permutation(n_out).astype(np.int32)
+    imap = rng.integers(0, n_in, n_out).astype(np.int32)
+    x = rng.standard_normal((n_in, c)).astype(dtype)
+    w = np.broadcast_to(np.eye(c, dtype=dtype), (k_vol, c, c)).copy()
+    D = dict(in_feats=torch.from_numpy(x).cuda(), kernel=torch.from_numpy(w).cuda(),
+             kpos=torch.from_numpy(kpos).cuda(), imap=torch.from_numpy(imap).cuda(),
+             omap=torch.from_numpy(omap).cuda(), n_in=n_in, n_out=n_out, c_in=c, c_out=c,
+             knnz_host=torch.from_numpy(knnz))
+    want = np.zeros((n_out, c), dtype)
+    want[omap] = x[imap]
+    for policy in (0, 1, 2):
+        capi.set_kernel_policy(policy)
+        for use_plan in (False, True):
+            plan = capi.Plan(D["kpos"], D["imap"], D["omap"], n_in, n_out) if use_plan else None
+            for fused in (True, False):
+                got = G.run_fwd(capi, D, fused=fused, plan=plan)
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (policy, use_plan, fused)
+    capi.set_kernel_policy(0)
+
+
+def test_duplicate_rows_inside_an_offset(capi, oracle):
+    """Not a sparse-conv map (an offset hits one output row twice): the plan
+    reports itself unusable and the atomic kernels still give the right sums."""
+    rng = np.random.default_rng(19)
+    n_in, n_out, k_vol = 900, 300, 3
+    knnz = np.array([500, 0, 700], np.int32)
+    kpos = np.concatenate([[0], np.cumsum(knnz)]).astype(np.int32)
+    imap = rng.integers(0, n_in, 1200).astype(np.int32)
+    omap = rng.integers(0, n_out, 1200).astype(np.int32)
+    L = clouds.make_layer(rng, imap, omap, knnz, kpos, n_in, n_out, 64, 64, np.float32)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], n_in, n_out)
+    assert not plan.usable(False) and not plan.usable(True)
+    G.assert_close(G.run_fwd(capi, D, plan=plan), oracle.np_fwd(L["in_feats"], L["kernel"], knnz, imap, omap, n_out), "fp32")
+    gi, gw = G.run_bwd(capi, D, plan=plan)
+    G.assert_close(gi, oracle.np_dgrad(L["out_grad"], L["kernel"], knnz, imap, omap, n_in), "fp32")
+    G.assert_close(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], knnz, imap, omap, k_vol), "fp32")
+
+
+def test_out_of_range_map_is_rejected_by_plan(capi):
+    kpos = torch.tensor([0, 2, 4], dtype=torch.int32, device="cuda")
+    imap = torch.tensor([0, 1, 2, 99], dtype=torch.int32, device="cuda")
+    omap = torch.tensor([0, 1, 2, 3], dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="outside"):
+        capi.Plan(kpos, imap, omap, 10, 10)
+
+
+def test_empty_inputs(capi):
+    for dtype in (torch.float32, torch.float16):
+        x = torch.randn(10, 32, device="cuda").to(dtype)
+        w = torch.randn(27, 32, 32, device="cuda").to(dtype)
+        out = torch.zeros(10, 32, device="cuda", dtype=dtype)
+        kpos = torch.zeros(28, dtype=torch.int32, device="cuda")
+        e = torch.zeros(0, dtype=torch.int32, device="cuda")
+        capi.fusion_fwd(x, w, 0, out, kpos, kpos, e, e, False, False)
+        capi.seq_fwd(x, w, 0, out, torch.zeros(27, dtype=torch.int32), kpos, e, e, False, False)
+        gi, gw = torch.zeros_like(x), torch.zeros_like(w)
+        capi.bwd(out, x, w, 0, gi, gw, kpos, kpos, e, e, False, False)
+        plan = capi.Plan(kpos, e, e, 10, 10)
+        capi.fusion_fwd(x, w, 0, out, kpos, kpos, e, e, False, False, plan=plan)
+        torch.cuda.synchronize()
+        assert not out.any() and not gi.any() and not gw.any()
+    with pytest.raises(ValueError):
+        capi.fusion_fwd(x, w[:, :16], 0, out, kpos, kpos, e, e, False, False)
+
+
+@pytest.mark.parametrize("cfg,variant", [(1, None), (3, None), (4, None), (4, "up"), (5, "skinny"), (5, "wide")])
+def test_baseline_configs_scaled(capi, oracle, cfg, variant):
+    """The benchmark configurations at a size the oracle finishes in seconds."""
+    L = clouds.config_case(cfg, variant, scale=0.08 if cfg != 1 else 0.5)
+    check_all(capi, oracle, L, policy=0, use_plan=True)
+    check_all(capi, oracle, L, policy=0, use_plan=False)
+
+
+def test_config2_scaled_fp32_and_tf32(capi, oracle):
+    L = clouds.config_case(2, scale=0.08)
+    check_all(capi, oracle, L, policy=0, use_plan=True, arch80=False)
+    check_all(capi, oracle, L, policy=0, use_plan=True, arch80=True)
