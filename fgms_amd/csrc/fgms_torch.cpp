@@ -12,9 +12,8 @@
 //  * HIP errors raise RuntimeError instead of passing silently.
 #include <torch/extension.h>
 
-#include <ATen/hip/HIPContext.h>
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <cstdlib>
 #include <list>
@@ -128,8 +127,8 @@ void ConvolutionForwardFused(const at::Tensor in_feats, const at::Tensor kernel,
   need_contiguous_cuda(out_feats, "out_feats"); need_contiguous_cuda(kpos, "kpos");
   need_contiguous_cuda(in_map, "in_map"); need_contiguous_cuda(out_map, "out_map");
   same_dtype(in_feats, kernel, "kernel"); same_dtype(in_feats, out_feats, "out_feats");
-  c10::hip::HIPGuard guard(in_feats.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(in_feats.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   const int k_vol = (int)kernel.size(0);
   fgms_plan_t *plan = plan_for(kpos, in_map, out_map, in_feats.size(0), out_feats.size(0), k_vol, stream);
   check(fgms_fusion_fwd(in_feats.data_ptr(), kernel.data_ptr(), sum_nnz, out_feats.data_ptr(),
@@ -153,8 +152,8 @@ void ConvolutionForward(const at::Tensor in_feats, const at::Tensor kernel, cons
   const int k_vol = (int)kernel.size(0);
   if (kernel_nnz.numel() < k_vol) throw std::invalid_argument("kernel_nnz is shorter than k_vol");
   at::Tensor knnz = kernel_nnz.contiguous();
-  c10::hip::HIPGuard guard(in_feats.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(in_feats.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   fgms_plan_t *plan = plan_for(kernel_pos, in_map, out_map, in_feats.size(0), out_feats.size(0), k_vol, stream);
   check(fgms_fwd(in_feats.data_ptr(), kernel.data_ptr(), sum_nnz, out_feats.data_ptr(),
                  knnz.data_ptr<int>(), i32(kernel_pos), i32(in_map), i32(out_map), separate_mid,
@@ -174,8 +173,8 @@ void ConvolutionBackward(const at::Tensor out_feats_grad, const at::Tensor in_fe
   need_contiguous_cuda(in_map, "in_map"); need_contiguous_cuda(out_map, "out_map");
   same_dtype(in_feats, kernel, "kernel"); same_dtype(in_feats, out_feats_grad, "out_feats_grad");
   same_dtype(in_feats, in_feats_grad, "in_feats_grad"); same_dtype(in_feats, kernel_grad, "kernel_grad");
-  c10::hip::HIPGuard guard(in_feats.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(in_feats.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   const int k_vol = (int)kernel.size(0);
   fgms_plan_t *plan = plan_for(kpos, in_map, out_map, in_feats.size(0), out_feats_grad.size(0), k_vol, stream);
   check(fgms_bwd(out_feats_grad.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), sum_nnz,
