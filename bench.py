@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused gather-GEMM-scatter path on one MI355X.
+
+Default workload (the one the headline metric is quoted on): the indoor-like
+cloud of ~200 k voxels, 27 offsets, 64 -> 64 channels, fp16, one step =
+forward + input gradient + weight gradient.  The protocol follows the
+reference's timing script (10 warm-up + 100 timed calls, spconv-test.py:95-122).
+
+Prints ONE JSON line:  effective TFLOP/s = passes * 2 * M * Cin * Cout / t with
+M the real (unpadded) pair count, a roofline object for the dominant kernel
+(duration from HIP events on the launch stream) and the CPU baseline (the C
+restatement of cpu-check.py / cpu-check-back.py on this box's host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3}
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (config id, variant, passes)
+    "cfg2-indoor200k-k27-64x64-fp16-fwd+dgrad+wgrad": (2, "fp16", ("fwd", "dgrad", "wgrad")),
+    "cfg2-indoor200k-k27-64x64-fp16-fwd": (2, "fp16", ("fwd",)),
+    "cfg2-indoor200k-k27-64x64-fp32-fwd": (2, None, ("fwd",)),
+    "cfg2-indoor200k-k27-64x64-tf32-fwd": (2, "tf32", ("fwd",)),
+    "cfg1-planes20k-k27-32x32-fp32-fwd+dgrad+wgrad": (1, None, ("fwd", "dgrad", "wgrad")),
+    "cfg3-lidar120k-k27-128x128-fp16-fwd+dgrad+wgrad": (3, None, ("fwd", "dgrad", "wgrad")),
+    "cfg4-down-k8-64x128-fp16-fwd+dgrad+wgrad": (4, None, ("fwd", "dgrad", "wgrad")),
+    "cfg4-up-k8-128x64-fp16-fwd+dgrad+wgrad": (4, "up", ("fwd", "dgrad", "wgrad")),
+    "cfg5-skinny-k27-4x32-fp16-fwd": (5, "skinny", ("fwd",)),
+    "cfg5-skinny-k27-4x32-fp32-fwd": (5, "skinny-fp32", ("fwd",)),
+    "cfg5-wide50k-k27-256x256-fp16-fwd": (5, "wide", ("fwd",)),
+    "cfg5-wide50k-k27-256x256-fp32-fwd": (5, "wide-fp32", ("fwd",)),
+}
+DEFAULT = "cfg2-indoor200k-k27-64x64-fp16-fwd+dgrad+wgrad"
+
+
+def make_case(name, scale=1.0):
+    import numpy as np
+    from fgms_amd import clouds
+    cfg, variant, passes = WORKLOADS[name]
+    arch80 = variant == "tf32"
+    L = clouds.config_case(cfg, None if variant == "tf32" else variant, scale=scale)
+    return L, passes, arch80
+
+
+def dataflow_bytes(L, which):
+    """Bytes one pass moves if every gathered row is read once per pair and every
+    result row written once per pair (the pair-list dataflow), plus maps and
+    weights: M*(Cin+Cout)*s + 8*M + K*Cin*Cout*s."""
+    s = L["in_feats"].dtype.itemsize
+    m = len(L["imap"])
+    return m * (L["c_in"] + L["c_out"]) * s + 8 * m + L["k_vol"] * L["c_in"] * L["c_out"] * s
+
+
+def cpu_baseline(name, budget_s=15.0):
+    """Times the CPU oracle (OpenMP, this box's host cores) on a bounded sample of
+    the same workload and returns effective TFLOP/s."""
+    from oracle import fgms_oracle as oracle
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    threads = max(1, min(threads, oracle.max_threads() if oracle.max_threads() > 0 else threads))
+
+    def run(scale):
+        L, passes, _ = make_case(name, scale)
+        args = (L["knnz"], L["imap"], L["omap"])
+        t0 = time.perf_counter()
+        if "fwd" in passes:
+            oracle.c_fwd(L["in_feats"], L["kernel"], *args, L["n_out"], threads=threads)
+        if "dgrad" in passes:
+            oracle.c_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"], threads=threads)
+        if "wgrad" in passes:
+            oracle.c_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"], threads=threads)
+        dt = time.perf_counter() - t0
+        flops = len(passes) * 2.0 * len(L["imap"]) * L["c_in"] * L["c_out"]
+        return dt, flops, L
+
+    scale = 0.05
+    dt, flops, L = run(scale)          # probe, then a sample sized to the budget
+    want = min(1.0, scale * budget_s / max(dt, 1e-3))
+    if want > 1.2 * scale:
+        scale = want
+        dt, flops, L = run(scale)
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": "%s at %.0f%% of the voxels (%d voxels, %d pairs), one pass each of %s, %.1f s"
+                  % (name.split("-")[0] + " cloud", scale * 100, L["n_in"], len(L["imap"]),
+                     "+".join(WORKLOADS[name][2]), dt),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--policy", type=int, default=0, help="0 auto, 1 generic kernels, 2 pair-stationary MFMA")
+    ap.add_argument("--no-plan", action="store_true", help="do not pass a kernel-map plan")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--scale", type=float, default=1.0, help="voxel-count scale (1.0 = the named size)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (every figure is "
+              "the single-GPU throughput at the full shape)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from fgms_amd import capi
+    from tests.gpu_util import to_dev
+
+    capi.lib()  # fails loudly if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    L, passes, arch80 = make_case(args.workload, args.scale)
+    D = to_dev(L)
+    capi.set_kernel_policy(args.policy)
+    plan = None if args.no_plan else capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    dt = D["in_feats"].dtype
+    out = torch.zeros(D["n_out"], D["c_out"], dtype=dt, device="cuda")
+    gi = torch.zeros(D["n_in"], D["c_in"], dtype=dt, device="cuda")
+    gw = torch.zeros_like(D["kernel"])
+    m = len(L["imap"])
+    flops_pass = 2.0 * m * L["c_in"] * L["c_out"]
+
+    def step():
+        if "fwd" in passes:
+            capi.fusion_fwd(D["in_feats"], D["kernel"], 0, out, D["kpos"], None, D["imap"], D["omap"],
+                            False, arch80, plan=plan)
+        if "dgrad" in passes:
+            capi.dgrad(D["out_grad"], D["kernel"], gi, D["kpos"], D["imap"], D["omap"], plan=plan)
+        if "wgrad" in passes:
+            capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
+
+    for _ in range(args.warmup):
+        step()
+    out.zero_(); gi.zero_(); gw.zero_()
+    torch.cuda.synchronize()
+    capi.profile_reset()
+    capi.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    capi.profile_enable(False)
+    recs = capi.profile_records()
+    capi.profile_reset()
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = len(passes) * flops_pass / (ms_per_step * 1e-3) / 1e12
+
+    # per-kernel averages from the HIP events recorded on the launch stream
+    per = {}
+    for name, ms in recs:
+        per.setdefault(name, []).append(ms)
+    kernels = {k: {"launches": len(v), "avg_ms": sum(v) / len(v)} for k, v in per.items()}
+    arith = "f16" if dt == torch.float16 else "f32"
+    roofline = None
+    if kernels:
+        dom = max(kernels, key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches"])
+        avg_s = kernels[dom]["avg_ms"] * 1e-3
+        skinny = min(L["c_in"], L["c_out"]) <= 16
+        if skinny:
+            which = "dgrad" if "dgrad" in dom else "fwd"
+            ach = dataflow_bytes(L, which) / avg_s / 1e9
+            roofline = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
+                        "avg_kernel_ms": kernels[dom]["avg_ms"]}
+        else:
+            ach = flops_pass / avg_s / 1e12
+            roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_TFLOPS[arith],
+                        "unit": "TFLOP/s", "frac": ach / PEAK_TFLOPS[arith], "traffic": None,
+                        "avg_kernel_ms": kernels[dom]["avg_ms"]}
+
+    line = {
+        "metric": "effective TFLOP/s (2*sum|map_k|*Cin*Cout/t), %s, %s"
+                  % ("+".join(passes), "tf32 mode" if arch80 else ("fp16" if arith == "f16" else "fp32")),
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": arith, "data": "synthetic",
+        "config": {"workload": args.workload, "voxels_in": L["n_in"], "voxels_out": L["n_out"],
+                   "pairs": m, "k_vol": L["k_vol"], "c_in": L["c_in"], "c_out": L["c_out"],
+                   "plan": plan is not None, "policy": args.policy},
+        "kernels": kernels,
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -16,7 +16,8 @@ F32, F16 = 0, 1
 SYMBOLS = [
     "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
-    "fgms_wgrad", "fgms_set_kernel_policy",
+    "fgms_wgrad", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
+    "fgms_profile_reset",
 ]
 
 _lib = None
@@ -51,6 +52,10 @@ def lib():
     L.fgms_wgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_set_kernel_policy.argtypes = [i32]
     L.fgms_set_kernel_policy.restype = None
+    L.fgms_profile_enable.argtypes = [i32]
+    L.fgms_profile_enable.restype = None
+    L.fgms_profile_reset.restype = None
+    L.fgms_profile_read.argtypes = [i32, ctypes.c_char_p, i32, ctypes.POINTER(ctypes.c_float)]
     _lib = L
     return L
 
@@ -93,6 +98,26 @@ def _need(t, name, dtype=None):
 def set_kernel_policy(policy):
     """0 automatic, 1 generic kernels only, 2 pair-stationary MFMA even with a plan."""
     lib().fgms_set_kernel_policy(int(policy))
+
+
+def profile_enable(on=True):
+    lib().fgms_profile_enable(int(on))
+
+
+def profile_reset():
+    lib().fgms_profile_reset()
+
+
+def profile_records():
+    """[(kernel name, milliseconds)] of every main-kernel launch since the last
+    reset, timed with HIP events on the launch stream."""
+    out, i = [], 0
+    name = ctypes.create_string_buffer(96)
+    ms = ctypes.c_float()
+    while lib().fgms_profile_read(i, name, 96, ctypes.byref(ms)) == 0:
+        out.append((name.value.decode(), float(ms.value)))
+        i += 1
+    return out
 
 
 class Plan:

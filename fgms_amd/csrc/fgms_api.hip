@@ -6,6 +6,8 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
+#include <string.h>
 
 #include "fgms_internal.h"
 
@@ -64,6 +66,33 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr) {
   }
   *ptr = b.ptr;
   return FGMS_OK;
+}
+
+// ---- profiling records -------------------------------------------------------
+namespace {
+struct ProfRec {
+  const char *name;
+  hipEvent_t start, stop;
+};
+std::mutex g_prof_mutex;
+std::vector<ProfRec> g_prof;
+bool g_prof_on = false;
+}  // namespace
+
+ProfileScope::ProfileScope(const char *name, hipStream_t s) : slot(-1), stream(s) {
+  if (!g_prof_on) return;
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  ProfRec r{name, nullptr, nullptr};
+  if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) return;
+  (void)hipEventRecord(r.start, stream);
+  g_prof.push_back(r);
+  slot = (int)g_prof.size() - 1;
+}
+
+ProfileScope::~ProfileScope() {
+  if (slot < 0) return;
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  if (slot < (int)g_prof.size()) (void)hipEventRecord(g_prof[slot].stop, stream);
 }
 
 namespace {
@@ -139,6 +168,30 @@ extern "C" {
 const char *fgms_version(void) { return "fgms-hip 0.1 (gfx950)"; }
 const char *fgms_last_error(void) { return g_error; }
 void fgms_set_kernel_policy(int policy) { g_policy = policy; }
+
+void fgms_profile_enable(int on) { g_prof_on = on != 0; }
+
+void fgms_profile_reset(void) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  for (auto &r : g_prof) {
+    (void)hipEventSynchronize(r.stop);
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_prof.clear();
+}
+
+int fgms_profile_read(int index, char *name, int name_len, float *ms) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  if (index < 0 || index >= (int)g_prof.size() || !ms) return FGMS_E_INVALID;
+  FGMS_HIP_TRY(hipEventSynchronize(g_prof[index].stop));
+  FGMS_HIP_TRY(hipEventElapsedTime(ms, g_prof[index].start, g_prof[index].stop));
+  if (name && name_len > 0) {
+    strncpy(name, g_prof[index].name, (size_t)name_len - 1);
+    name[name_len - 1] = 0;
+  }
+  return FGMS_OK;
+}
 
 int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_feats,
                     const int32_t *kpos, const int32_t *qkpos, const int32_t *in_map,

@@ -187,6 +187,7 @@ int launch_generic_gms(const GmsArgs &a) {
   else tiles = (a.n_pairs + kRows - 1) / kRows + a.k_vol;
   if (tiles <= 0) return FGMS_OK;
   dim3 grid((unsigned)tiles, (unsigned)((c_dst + kCols - 1) / kCols));
+  ProfileScope prof(a.transpose_w ? "generic_gms_kernel(dgrad)" : "generic_gms_kernel(fwd)", a.stream);
   if (a.dtype == FGMS_F16) {
     generic_gms_kernel<__half><<<grid, kThreads, 0, a.stream>>>(
         (const __half *)a.src, (const __half *)a.w, (__half *)a.dst, a.kpos, a.gmap, a.smap,
@@ -219,12 +220,16 @@ int launch_generic_wgrad(const WgradArgs &a) {
   const int ty = ((a.c_in + kTile - 1) / kTile) * ((a.c_out + kTile - 1) / kTile);
   dim3 grid((unsigned)tiles, (unsigned)ty);
   if (a.dtype == FGMS_F16) {
-    generic_wgrad_kernel<__half><<<grid, kThreads, 0, a.stream>>>(
-        (const __half *)a.in, (const __half *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol,
-        a.c_in, a.c_out);
+    {
+      ProfileScope prof("generic_wgrad_kernel", a.stream);
+      generic_wgrad_kernel<__half><<<grid, kThreads, 0, a.stream>>>(
+          (const __half *)a.in, (const __half *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol,
+          a.c_in, a.c_out);
+    }
     add_from_f32_kernel<__half><<<(unsigned)((n + 255) / 256), 256, 0, a.stream>>>(
         (__half *)a.gw, acc32, n);
   } else {
+    ProfileScope prof("generic_wgrad_kernel", a.stream);
     generic_wgrad_kernel<float><<<grid, kThreads, 0, a.stream>>>(
         (const float *)a.in, (const float *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol,
         a.c_in, a.c_out);

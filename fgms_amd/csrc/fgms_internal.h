@@ -66,8 +66,8 @@ struct Plan {
   int device;
   int k_vol;
   int64_t n_in, n_out, n_pairs;
-  int32_t *nbr_out;   // [n_out, k_vol]: input row feeding output row o through offset k, or -1
-  int32_t *nbr_in;    // [n_in,  k_vol]: output row fed by input row i through offset k, or -1
+  int32_t *nbr_out;   // [k_vol, n_out]: input row feeding output row o through offset k, or -1
+  int32_t *nbr_in;    // [k_vol, n_in]:  output row fed by input row i through offset k, or -1
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -75,6 +75,14 @@ struct Plan {
 // Fp32 scratch that outlives a call (per device and stream, grown on demand).
 // slot 0: packed weights, slot 1: fp32 weight-gradient accumulator.
 int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr);
+
+// Brackets a main-kernel launch with events when profiling is enabled.
+struct ProfileScope {
+  ProfileScope(const char *name, hipStream_t stream);
+  ~ProfileScope();
+  int slot;
+  hipStream_t stream;
+};
 
 // ---- launchers (each returns an FGMS_* code) ----
 int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);

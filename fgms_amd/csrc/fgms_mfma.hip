@@ -1,10 +1,517 @@
-// placeholder: MFMA kernels
+// MFMA gather-GEMM-scatter kernels for gfx950 (forward and input gradient).
+//
+// Two dataflows share one fragment scheme:
+//
+//  * pair-stationary ("pairs"): a workgroup walks a run of 256-pair tiles of the
+//    flat pair list, keeps op(W[k]) in LDS while the offset k does not change,
+//    gathers the source rows through LDS and scatters the products with
+//    atomics.  Works for any map.  This is the dataflow of the reference's fused
+//    kernels (backend/spconv.cuh:1328-1477, backend/fwd_kernels.cuh:17-144,
+//    backend/bwd_kernels.cuh:13-142, 281-408) re-tiled for 64-wide waves.
+//  * output-stationary ("rows"): a workgroup owns 256 destination rows, walks the
+//    offsets k through the plan's neighbour table, sums everything in MFMA
+//    accumulators and writes each destination row once: no atomics, run-to-run
+//    identical results.  Needs a plan whose map is functional.
+//
+// Fragment scheme.  A source row is cut into slabs of 2*S 16-byte chunks
+// (S = 4, 2 or 1; a chunk is 8 halfs or 4 floats).  Lanes 0-31 of a wave carry
+// the first S chunks of the slab, lanes 32-63 the last S, so one MFMA
+// (v_mfma_f32_32x32x16_f16, or four v_mfma_f32_32x32x2_f32) contracts chunk s of
+// both halves.  The order of the contraction index is free as long as both
+// operands agree, and it lets every lane read one contiguous 16-byte piece.
+// Weights are re-laid on the device into exactly that per-lane order before the
+// main kernel runs (pack_weights_kernel), transposed for the input gradient.
+//
+// Gathered rows reach LDS with 16-byte loads, 2*S lanes per row (full 128-byte
+// lines for S = 4), in an XOR-swizzled layout so that the b128 reads of the MFMA
+// operand do not collide on banks.
+#include <type_traits>
+
+#include "fgms_device.h"
 #include "fgms_internal.h"
+
 namespace fgms {
-bool mfma_gms_supported(const GmsArgs &) { return false; }
-int launch_mfma_gms(const GmsArgs &) { return FGMS_E_INVALID; }
-bool mfma_wgrad_supported(const WgradArgs &) { return false; }
-int launch_mfma_wgrad(const WgradArgs &) { return FGMS_E_INVALID; }
-bool planned_gms_supported(const GmsArgs &, const Plan *) { return false; }
-int launch_planned_gms(const GmsArgs &, const Plan *) { return FGMS_E_INVALID; }
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kWaveRows = 64;                 // two 32-row MFMA tiles per wave
+constexpr int kTileRows = kWaves * kWaveRows; // 256 rows per workgroup tile
+
+template <typename T> struct Elem;
+template <> struct Elem<__half> { static constexpr int per_chunk = 8; };
+template <> struct Elem<float> { static constexpr int per_chunk = 4; };
+
+template <typename T>
+__device__ __forceinline__ void mma(float16v &acc, const int4v &a, const int4v &b) {
+  if constexpr (sizeof(T) == 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a),
+                                                 __builtin_bit_cast(half8, b), acc, 0, 0, 0);
+  } else {
+    const float4v fa = __builtin_bit_cast(float4v, a), fb = __builtin_bit_cast(float4v, b);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1], fb[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2], fb[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[3], fb[3], acc, 0, 0, 0);
+  }
 }
+
+// LDS ordering between lanes of one wave: LDS operations of a wave complete in
+// program order; the fence keeps the compiler from moving them across.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// Slot of 16-byte chunk c of row `row` inside a wave's staging tile
+// (rows of 2*S chunks).  8 consecutive slots cover all LDS banks once; the XOR
+// spreads the 8 rows that one b128 read pass touches over distinct slots.
+template <int S>
+__device__ __forceinline__ int a_slot(int row, int c) {
+  constexpr int C = 2 * S;
+  return row * C + (c ^ ((row / (8 / C)) % C));
+}
+
+// ---------------------------------------------------------------------------
+// Weight re-layout.  packed[k][q][nt][lane][e], q = slab * S + s:
+//   source channel  cs = slab * 2*S*E + (lane / 32) * S*E + s * E + e
+//   dest   channel  cd = nt * 32 + lane % 32
+//   value = transpose ? W[k][cd][cs] : W[k][cs][cd]
+template <typename T>
+__global__ void pack_weights_kernel(const T *__restrict__ w, T *__restrict__ packed, int k_vol,
+                                    int c_in, int c_out, int S, bool transpose) {
+  constexpr int E = Elem<T>::per_chunk;
+  const int c_src = transpose ? c_out : c_in;
+  const int c_dst = transpose ? c_in : c_out;
+  const size_t per_k = (size_t)c_src * c_dst;
+  const size_t total = per_k * k_vol;
+  const int nts = c_dst / 32;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (size_t)gridDim.x * blockDim.x) {
+    const int k = (int)(i / per_k);
+    size_t r = i % per_k;
+    const int e = (int)(r % E); r /= E;
+    const int lane = (int)(r % 64); r /= 64;
+    const int nt = (int)(r % nts); r /= nts;
+    const int q = (int)r;
+    const int slab = q / S, s = q % S;
+    const int cs = slab * 2 * S * E + (lane / 32) * S * E + s * E + e;
+    const int cd = nt * 32 + lane % 32;
+    const T *wk = w + (size_t)k * c_in * c_out;
+    packed[i] = transpose ? wk[(size_t)cd * c_out + cs] : wk[(size_t)cs * c_out + cd];
+  }
+}
+
+// Copies the packed weights of offset k, destination tiles [nt0, nt0 + NT), to LDS.
+template <int NT>
+__device__ __forceinline__ void load_weights(int4v *__restrict__ w_lds,
+                                             const int4v *__restrict__ packed_k, int qs, int nts,
+                                             int nt0) {
+  const int n = qs * NT * 64;
+  for (int i = threadIdx.x; i < n; i += kThreads) {
+    const int q = i / (NT * 64), rem = i % (NT * 64);
+    w_lds[i] = packed_k[((size_t)q * nts + nt0) * 64 + rem];
+  }
+}
+
+// Gathers one slab of the wave's 64 rows into its LDS staging tile.
+template <typename T, int S>
+__device__ __forceinline__ void stage_rows(int4v *__restrict__ a_lds, const int *__restrict__ idx,
+                                           const T *__restrict__ src, int c_src, int slab,
+                                           int lane) {
+  constexpr int E = Elem<T>::per_chunk;
+  constexpr int C = 2 * S;
+  int4v v[C];
+  int g[C];
+#pragma unroll
+  for (int it = 0; it < C; ++it) g[it] = idx[(it * 64 + lane) / C];
+  // every lane loads (absent rows read row 0 and are zeroed afterwards): no
+  // branch between the loads, so all of them are in flight together
+#pragma unroll
+  for (int it = 0; it < C; ++it) {
+    const int c = (it * 64 + lane) % C;
+    v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(g[it], 0) * c_src +
+                                             (size_t)(slab * C + c) * E);
+  }
+#pragma unroll
+  for (int it = 0; it < C; ++it)
+    if (g[it] < 0) v[it] = int4v{0, 0, 0, 0};
+#pragma unroll
+  for (int it = 0; it < C; ++it) {
+    const int slot = it * 64 + lane;
+    a_lds[a_slot<S>(slot / C, slot % C)] = v[it];
+  }
+}
+
+// acc[mt][nt] += A(slab) x W(slab).
+template <typename T, int NT, int S>
+__device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+                                         const int4v *__restrict__ w_lds, int slab, int lane) {
+  const int h = lane / 32, r = lane % 32;
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    int4v b[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[((slab * S + s) * NT + nt) * 64 + lane];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+    }
+  }
+}
+
+__device__ __forceinline__ float swap_with_neighbour(float v) {
+  // lane ^ 1 inside each quad: quad_perm [1, 0, 3, 2]
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+}
+
+// Writes a wave's accumulators.  Accumulator register r of lane l holds row
+// (r / 4) * 8 + (l / 32) * 4 + r % 4 and column l % 32 of its 32x32 tile.  For
+// fp16 two lanes swap one value each so that every lane owns two neighbouring
+// columns of one row and can issue a packed 4-byte update.
+template <typename T, int NT, bool ATOMIC>
+__device__ __forceinline__ void write_tile(const float16v (&acc)[2][NT], T *__restrict__ dst,
+                                           const int *__restrict__ rows, int c_dst, int cd0,
+                                           int lane) {
+  const int h = lane / 32, col = lane % 32;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = rows[mt * 32 + (r / 4) * 8 + h * 4 + (r % 4)];
+          if (row >= 0) {
+            float *p = reinterpret_cast<float *>(dst) + (size_t)row * c_dst + cd0 + nt * 32 + col;
+            if constexpr (ATOMIC) atomic_add(p, acc[mt][nt][r]);
+            else *p += acc[mt][nt][r];
+          }
+        }
+      } else {
+        const bool odd = col & 1;
+#pragma unroll
+        for (int rp = 0; rp < 8; ++rp) {
+          const float v0 = acc[mt][nt][2 * rp], v1 = acc[mt][nt][2 * rp + 1];
+          const float got = swap_with_neighbour(odd ? v0 : v1);
+          const float lo = odd ? got : v0, hi = odd ? v1 : got;
+          const int r = 2 * rp + (odd ? 1 : 0);
+          const int row = rows[mt * 32 + (r / 4) * 8 + h * 4 + (r % 4)];
+          if (row >= 0) {
+            __half *p = reinterpret_cast<__half *>(dst) + (size_t)row * c_dst + cd0 + nt * 32 + (col & ~1);
+            if constexpr (ATOMIC) {
+              atomic_add_pk(p, lo, hi);
+            } else {
+              __half2 *q = reinterpret_cast<__half2 *>(p);
+              const float2 old = __half22float2(*q);
+              *q = __floats2half2_rn(old.x + lo, old.y + hi);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Pair-stationary kernel.
+template <typename T, int NT, int S>
+__global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
+    const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
+    const int32_t *__restrict__ kpos, const int32_t *__restrict__ gmap,
+    const int32_t *__restrict__ smap, int k_vol, int c_src, int c_dst, int tiles_per_wg,
+    int dense_k, int dense_rows) {
+  constexpr int E = Elem<T>::per_chunk;
+  extern __shared__ int4v lds[];
+  const int slabs = c_src / (2 * S * E);
+  const int qs = slabs * S;
+  const int nts = c_dst / 32;
+  int4v *w_lds = lds;                                   // qs * NT * 64 chunks
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  int4v *a_lds = lds + qs * NT * 64 + wave * (kWaveRows * 2 * S);
+  int *idx_all = reinterpret_cast<int *>(lds + qs * NT * 64 + kWaves * (kWaveRows * 2 * S));
+  int *gidx = idx_all + wave * 2 * kWaveRows;
+  int *sidx = gidx + kWaveRows;
+  const int nt0 = blockIdx.y * NT;
+  const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
+
+  int cur_k = -1;
+  const int t_begin = blockIdx.x * tiles_per_wg;
+  for (int t = t_begin; t < t_begin + tiles_per_wg; ++t) {
+    int k, first, count;
+    if (dense_k >= 0) {
+      k = dense_k;
+      first = t * kTileRows;
+      if (first >= dense_rows) break;
+      count = min(kTileRows, dense_rows - first);
+    } else if (!locate_tile(kpos, k_vol, kTileRows, t, k, first, count)) {
+      break;
+    }
+    if (k != cur_k) {  // uniform over the workgroup
+      __syncthreads();
+      load_weights<NT>(w_lds, reinterpret_cast<const int4v *>(packed) + packed_per_k * k, qs, nts, nt0);
+      __syncthreads();
+      cur_k = k;
+    }
+    const int wfirst = wave * kWaveRows;
+    const int nrows = min(kWaveRows, count - wfirst);
+    if (nrows <= 0) continue;
+    const bool live = lane < nrows;
+    const int j = first + wfirst + lane;
+    gidx[lane] = !live ? -1 : (gmap ? gmap[j] : j);
+    sidx[lane] = !live ? -1 : (smap ? smap[j] : j);
+    wave_lds_fence();
+
+    float16v acc[2][NT];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
+
+    for (int slab = 0; slab < slabs; ++slab) {
+      stage_rows<T, S>(a_lds, gidx, src, c_src, slab, lane);
+      wave_lds_fence();
+      mma_slab<T, NT, S>(acc, a_lds, w_lds, slab, lane);
+      wave_lds_fence();
+    }
+    write_tile<T, NT, true>(acc, dst, sidx, c_dst, nt0 * 32, lane);
+    wave_lds_fence();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Output-stationary kernel.  nbr is the plan's table laid out [k_vol][n_dst]:
+// nbr[k][d] = source row that reaches destination row d through offset k, or -1.
+template <typename T, int NT, int S>
+__global__ __launch_bounds__(kThreads) void gms_rows_kernel(
+    const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
+    const int32_t *__restrict__ nbr, int n_dst, int k_vol, int c_src, int c_dst) {
+  constexpr int E = Elem<T>::per_chunk;
+  extern __shared__ int4v lds[];
+  __shared__ unsigned long long wg_mask;
+  const int slabs = c_src / (2 * S * E);
+  const int qs = slabs * S;
+  const int nts = c_dst / 32;
+  int4v *w_lds = lds;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  int4v *a_lds = lds + qs * NT * 64 + wave * (kWaveRows * 2 * S);
+  int *idx_all = reinterpret_cast<int *>(lds + qs * NT * 64 + kWaves * (kWaveRows * 2 * S));
+  int *gidx = idx_all + wave * 2 * kWaveRows;
+  int *didx = gidx + kWaveRows;
+  const int nt0 = blockIdx.y * NT;
+  const size_t packed_per_k = (size_t)c_src * c_dst / E;
+
+  const int row0 = blockIdx.x * kTileRows + wave * kWaveRows;
+  const int my_row = row0 + lane;
+  const bool in_range = my_row < n_dst;
+  didx[lane] = in_range ? my_row : -1;
+
+  // which offsets touch this wave's rows / this workgroup's rows
+  unsigned long long wave_mask = 0;
+  for (int k = 0; k < k_vol; ++k) {
+    const int g = in_range ? nbr[(size_t)k * n_dst + my_row] : -1;
+    if (__ballot(g >= 0)) wave_mask |= 1ull << k;
+  }
+  if (threadIdx.x == 0) wg_mask = 0;
+  __syncthreads();
+  if (lane == 0 && wave_mask) atomicOr(&wg_mask, wave_mask);
+  __syncthreads();
+  unsigned long long todo = wg_mask;
+
+  float16v acc[2][NT];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
+
+  while (todo) {
+    const int k = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    __syncthreads();  // everyone is done with the previous offset's weights
+    load_weights<NT>(w_lds, reinterpret_cast<const int4v *>(packed) + packed_per_k * k, qs, nts, nt0);
+    __syncthreads();
+    if (!((wave_mask >> k) & 1)) continue;
+    const int g = in_range ? nbr[(size_t)k * n_dst + my_row] : -1;
+    gidx[lane] = g;
+    wave_lds_fence();
+    for (int slab = 0; slab < slabs; ++slab) {
+      stage_rows<T, S>(a_lds, gidx, src, c_src, slab, lane);
+      wave_lds_fence();
+      mma_slab<T, NT, S>(acc, a_lds, w_lds, slab, lane);
+      wave_lds_fence();
+    }
+  }
+  if (wave_mask) {
+    wave_lds_fence();
+    write_tile<T, NT, false>(acc, dst, didx, c_dst, nt0 * 32, lane);
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct Shape {
+  int c_src, c_dst, S, NT, E;
+  size_t lds_bytes;
+  bool ok;
+};
+
+Shape shape_of(const GmsArgs &a) {
+  Shape s{};
+  s.c_src = a.transpose_w ? a.c_out : a.c_in;
+  s.c_dst = a.transpose_w ? a.c_in : a.c_out;
+  s.E = a.dtype == FGMS_F16 ? 8 : 4;
+  const size_t esz = a.dtype == FGMS_F16 ? 2 : 4;
+  s.ok = false;
+  if (s.c_dst % 32 != 0 || s.c_src % (2 * s.E) != 0) return s;
+  s.S = (s.c_src % (8 * s.E) == 0) ? 4 : (s.c_src % (4 * s.E) == 0) ? 2 : 1;
+  s.NT = (s.c_dst % 64 == 0) ? 2 : 1;
+  // rows are read with 16-byte loads and fp16 results written as 4-byte pairs
+  if (reinterpret_cast<uintptr_t>(a.src) % 16 || reinterpret_cast<uintptr_t>(a.dst) % 4) return s;
+  s.lds_bytes = (size_t)s.c_src * s.NT * 32 * esz           // weights of one offset
+                + (size_t)kWaves * kWaveRows * 2 * s.S * 16  // staging tiles
+                + (size_t)kWaves * 2 * kWaveRows * sizeof(int);
+  s.ok = s.lds_bytes <= 128 * 1024;
+  return s;
+}
+
+template <typename T>
+int pack_weights(const GmsArgs &a, const Shape &s, const T **packed) {
+  void *ws = nullptr;
+  const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+  int rc = workspace_get(a.stream, 0, n * sizeof(T), &ws);
+  if (rc != FGMS_OK) return rc;
+  unsigned blocks = (unsigned)((n + 255) / 256);
+  if (blocks > 4096) blocks = 4096;
+  pack_weights_kernel<T><<<blocks, 256, 0, a.stream>>>((const T *)a.w, (T *)ws, a.k_vol, a.c_in,
+                                                       a.c_out, s.S, a.transpose_w);
+  FGMS_HIP_TRY(hipGetLastError());
+  *packed = (const T *)ws;
+  return FGMS_OK;
+}
+
+int num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
+      cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+template <typename T, int NT, int S>
+int launch_pairs(const GmsArgs &a, const Shape &s) {
+  const T *packed = nullptr;
+  int rc = pack_weights<T>(a, s, &packed);
+  if (rc != FGMS_OK) return rc;
+  const bool dense = a.dense_k >= 0;
+  const int64_t tiles = dense ? (a.n_dense + kTileRows - 1) / kTileRows
+                              : (a.n_pairs + kTileRows - 1) / kTileRows + a.k_vol;
+  // a few workgroups per CU, each walking a contiguous run of tiles
+  const int64_t want_wgs = (int64_t)num_cus() * 8;
+  const int tiles_per_wg = (int)((tiles + want_wgs - 1) / want_wgs);
+  const unsigned gx = (unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg);
+  auto kern = gms_pairs_kernel<T, NT, S>;
+  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)s.lds_bytes));
+  {
+    ProfileScope prof(a.transpose_w ? "gms_pairs_kernel(dgrad)" : "gms_pairs_kernel(fwd)", a.stream);
+    kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_bytes, a.stream>>>(
+        (const T *)a.src, packed, (T *)a.dst, a.kpos, a.gmap, a.smap, a.k_vol, s.c_src, s.c_dst,
+        tiles_per_wg, a.dense_k, (int)a.n_dense);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
+template <typename T, int NT, int S>
+int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr) {
+  const T *packed = nullptr;
+  int rc = pack_weights<T>(a, s, &packed);
+  if (rc != FGMS_OK) return rc;
+  const unsigned gx = (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
+  if (gx == 0) return FGMS_OK;
+  auto kern = gms_rows_kernel<T, NT, S>;
+  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)s.lds_bytes));
+  {
+    ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
+    kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_bytes, a.stream>>>(
+        (const T *)a.src, packed, (T *)a.dst, nbr, (int)a.n_dst, a.k_vol, s.c_src, s.c_dst);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
+template <typename T, typename F>
+int dispatch_shape(const Shape &s, F &&f) {
+  if (s.NT == 2) {
+    if (s.S == 4) return f(std::integral_constant<int, 2>{}, std::integral_constant<int, 4>{});
+    if (s.S == 2) return f(std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+    return f(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+  }
+  if (s.S == 4) return f(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+  if (s.S == 2) return f(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
+  return f(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
+}
+
+}  // namespace
+
+bool mfma_gms_supported(const GmsArgs &a) { return shape_of(a).ok; }
+
+int launch_mfma_gms(const GmsArgs &a) {
+  const Shape s = shape_of(a);
+  if (!s.ok) {
+    set_error("launch_mfma_gms: unsupported shape");
+    return FGMS_E_INVALID;
+  }
+  if (a.dtype == FGMS_F16)
+    return dispatch_shape<__half>(s, [&](auto nt, auto sv) {
+      return launch_pairs<__half, decltype(nt)::value, decltype(sv)::value>(a, s);
+    });
+  return dispatch_shape<float>(s, [&](auto nt, auto sv) {
+    return launch_pairs<float, decltype(nt)::value, decltype(sv)::value>(a, s);
+  });
+}
+
+bool planned_gms_supported(const GmsArgs &a, const Plan *p) {
+  if (!p || a.dense_k >= 0 || a.k_vol > 64 || a.k_vol != p->k_vol) return false;
+  if (a.transpose_w) {
+    if (!p->dgrad_ok || a.n_dst != p->n_in || a.n_src != p->n_out) return false;
+  } else {
+    if (!p->fwd_ok || a.n_dst != p->n_out || a.n_src != p->n_in) return false;
+  }
+  return shape_of(a).ok;
+}
+
+int launch_planned_gms(const GmsArgs &a, const Plan *p) {
+  const Shape s = shape_of(a);
+  if (!s.ok || !planned_gms_supported(a, p)) {
+    set_error("launch_planned_gms: unsupported shape or plan");
+    return FGMS_E_INVALID;
+  }
+  const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
+  if (a.dtype == FGMS_F16)
+    return dispatch_shape<__half>(s, [&](auto nt, auto sv) {
+      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr);
+    });
+  return dispatch_shape<float>(s, [&](auto nt, auto sv) {
+    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr);
+  });
+}
+
+// weight gradient: see fgms_wgrad.hip
+}  // namespace fgms

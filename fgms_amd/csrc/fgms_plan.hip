@@ -1,7 +1,8 @@
 // Kernel-map plan: neighbour tables built on the device from the pair lists.
-// nbr_out[o][k] = the input row that reaches output row o through offset k
-// (-1 if none); nbr_in[i][k] = the output row that input row i reaches through
-// offset k.  The reference keeps only the pair lists and scatters with atomics
+// nbr_out[k][o] = the input row that reaches output row o through offset k
+// (-1 if none); nbr_in[k][i] = the output row that input row i reaches through
+// offset k.  Offset-major, so a wave reads the entries of its 64 consecutive
+// rows for one offset as one 256-byte line.  The reference keeps only the pair lists and scatters with atomics
 // (backend/spconv.cuh:457-563); the tables let a workgroup own a block of
 // output rows and sum all offsets in registers.
 #include "fgms_device.h"
@@ -38,8 +39,8 @@ __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
     flags[0] = 1;
     return;
   }
-  if (atomicCAS(&nbr_out[(size_t)o * k_vol + k], -1, i) != -1) flags[1] = 1;
-  if (atomicCAS(&nbr_in[(size_t)i * k_vol + k], -1, o) != -1) flags[2] = 1;
+  if (atomicCAS(&nbr_out[(size_t)k * n_out + o], -1, i) != -1) flags[1] = 1;
+  if (atomicCAS(&nbr_in[(size_t)k * n_in + i], -1, o) != -1) flags[2] = 1;
 }
 
 int fill_i32(int32_t *p, size_t n, int32_t v, hipStream_t s) {

@@ -133,6 +133,19 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
  * kernels even when a usable plan is passed.  Process-wide. */
 void fgms_set_kernel_policy(int policy);
 
+/*
+ * Per-kernel timing with HIP events on the stream the kernels are launched on
+ * (no counterpart in the reference, which times whole calls from python,
+ * spconv-test.py:95-122).  While enabled, every main kernel launch (not the
+ * small weight re-layout or zero-fill launches) is bracketed by two events.
+ * fgms_profile_read synchronises with the recorded events and returns the
+ * index-th record: kernel name and milliseconds; it returns FGMS_E_INVALID
+ * once index runs past the records.  fgms_profile_reset drops all records.
+ */
+void fgms_profile_enable(int on);
+int fgms_profile_read(int index, char *name, int name_len, float *ms);
+void fgms_profile_reset(void);
+
 #ifdef __cplusplus
 }
 #endif
