@@ -1,6 +1,298 @@
-// placeholder: MFMA weight-gradient kernels
+// MFMA weight-gradient kernel for gfx950.
+//
+//   dW[k][ci][co] += sum over the pairs j of offset k of in[imap[j]][ci] * gout[omap[j]][co]
+//
+// The contraction runs over pairs.  A workgroup takes a run of pairs of one
+// offset ("chunk") and a CI x CO tile of dW[k] (the whole matrix up to
+// 128 x 128), stages the gathered `in` rows and `gout` rows of 64 (fp16) or 32
+// (fp32) pairs at a time in LDS with 16-byte loads, double-buffered so the next
+// stage's gathers are in flight while the current one is multiplied, and keeps
+// the tile in MFMA accumulators until the chunk ends; one fp32 atomic flush per
+// workgroup.  Each row is gathered once per chunk, not once per 32x32 tile of dW
+// as in the reference (backend/bwd_kernels.cuh:935-954).
+//
+// fp16: both MFMA operands need 8 consecutive PAIRS of one channel per lane,
+// the transpose of how rows sit in LDS; ds_read_b64_tr_b16 does that transpose
+// on the way out of LDS (16 lanes hand in the addresses of a 4-row x 16-column
+// block, lane i gets column i).  fp32: v_mfma_f32_32x32x2_f32 takes one element
+// per lane, so plain ds_read_b32 along a row is already the right shape.
+#include <type_traits>
+
+#include "fgms_device.h"
 #include "fgms_internal.h"
+
 namespace fgms {
-bool mfma_wgrad_supported(const WgradArgs &) { return false; }
-int launch_mfma_wgrad(const WgradArgs &) { return FGMS_E_INVALID; }
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+
+template <typename T> struct WT;
+template <> struct WT<__half> {
+  static constexpr int E = 8;          // elements per 16-byte chunk
+  static constexpr int stage_pairs = 64;
+  static constexpr int step_pairs = 16; // pairs per k-step (one 32x32x16 MFMA)
+  static constexpr int pad = 16;        // row padding in elements (32 bytes)
+};
+template <> struct WT<float> {
+  static constexpr int E = 4;
+  static constexpr int stage_pairs = 32;
+  static constexpr int step_pairs = 8;  // four 32x32x2 MFMAs
+  static constexpr int pad = 4;
+};
+
+template <int BI, int BJ> struct WaveGrid {
+  static constexpr int WI = BI >= 2 ? (BJ == 1 && BI == 4 ? 4 : 2) : 1;
+  static constexpr int WJ = BJ >= 2 ? (BI == 1 && BJ == 4 ? 4 : (WI == 4 ? 1 : 2)) : 1;
+  static constexpr int WK = 4 / (WI * WJ);
+  static constexpr int TI = BI / WI;
+  static constexpr int TJ = BJ / WJ;
+  static_assert(WI * WJ * WK == 4 && TI * WI == BI && TJ * WJ == BJ, "wave grid");
+};
+
+// One k-step (16 pairs) of one 32-wide operand block, fp16: returns the 8
+// pair-values of channel (lane % 32) for pairs p0 + 8 * (lane / 32) + 0..7.
+__device__ __forceinline__ half8 tr_frag(const __half *tile, int ld, int p0, int c0, int lane) {
+  const int b = lane >> 4, i = lane & 15, h = lane >> 5;
+  const __half *base = tile + (size_t)(p0 + h * 8 + (i >> 2)) * ld + c0 + (b & 1) * 16 + (i & 3) * 4;
+  typedef __attribute__((address_space(3))) short4v lds_v4;
+  const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4 *)(base));
+  const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4 *)(base + 4 * ld));
+  const short8v v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(half8, v);
 }
+
+template <typename T, int BI, int BJ>
+__global__ __launch_bounds__(kThreads) void wgrad_kernel(
+    const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
+    const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk) {
+  using W = WT<T>;
+  using G = WaveGrid<BI, BJ>;
+  constexpr int E = W::E, SP = W::stage_pairs, KP = W::step_pairs;
+  constexpr int CI = BI * 32, CO = BJ * 32;
+  constexpr int LDI = CI + W::pad, LDO = CO + W::pad;
+  constexpr int NCI = CI / E, NCO = CO / E;   // 16-byte chunks per staged row
+  constexpr int NX = BI, NG = BJ;             // chunks per thread and stage
+  extern __shared__ int4v lds[];
+  T *xs[2], *gs[2];
+  xs[0] = reinterpret_cast<T *>(lds);
+  gs[0] = xs[0] + SP * LDI;
+  xs[1] = gs[0] + SP * LDO;
+  gs[1] = xs[1] + SP * LDI;
+
+  int k, first, count;
+  if (!locate_tile(kpos, k_vol, chunk, blockIdx.x, k, first, count)) return;
+  const int tiles_co = c_out / CO;
+  const int ci0 = (blockIdx.y / tiles_co) * CI;
+  const int co0 = (blockIdx.y % tiles_co) * CO;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int wi = wave % G::WI, wj = (wave / G::WI) % G::WJ, wk = wave / (G::WI * G::WJ);
+
+  float16v acc[G::TI][G::TJ];
+#pragma unroll
+  for (int a = 0; a < G::TI; ++a)
+#pragma unroll
+    for (int b = 0; b < G::TJ; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  const int nstages = (count + SP - 1) / SP;
+  int xi[NX], gi[NG];      // gather rows of the stage about to be loaded
+  int4v xr[NX], gr[NG];    // its data while in flight
+
+  auto load_idx = [&](int st) {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int p = st * SP + (tid + kThreads * i) / NCI;
+      xi[i] = p < count ? imap[first + p] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int p = st * SP + (tid + kThreads * i) / NCO;
+      gi[i] = p < count ? omap[first + p] : -1;
+    }
+  };
+  auto load_rows = [&]() {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int cc = (tid + kThreads * i) % NCI;
+      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)max(xi[i], 0) * c_in + ci0 + cc * E);
+    }
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int cc = (tid + kThreads * i) % NCO;
+      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)max(gi[i], 0) * c_out + co0 + cc * E);
+    }
+#pragma unroll
+    for (int i = 0; i < NX; ++i)
+      if (xi[i] < 0) xr[i] = int4v{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+      if (gi[i] < 0) gr[i] = int4v{0, 0, 0, 0};
+  };
+  auto store_rows = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int e = tid + kThreads * i;
+      *reinterpret_cast<int4v *>(xs[buf] + (e / NCI) * LDI + (e % NCI) * E) = xr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int e = tid + kThreads * i;
+      *reinterpret_cast<int4v *>(gs[buf] + (e / NCO) * LDO + (e % NCO) * E) = gr[i];
+    }
+  };
+
+  load_idx(0);
+  load_rows();
+  store_rows(0);
+  if (nstages > 1) load_idx(1);
+  __syncthreads();
+
+  for (int st = 0; st < nstages; ++st) {
+    const int cur = st & 1;
+    const bool more = st + 1 < nstages;
+    if (more) {
+      load_rows();                          // stage st + 1, in flight during the MFMAs
+      if (st + 2 < nstages) load_idx(st + 2);
+    }
+    const T *x = xs[cur], *g = gs[cur];
+#pragma unroll
+    for (int ks = wk; ks < SP / KP; ks += G::WK) {
+      const int p0 = ks * KP;
+      if constexpr (sizeof(T) == 2) {
+        half8 a[G::TI], b[G::TJ];
+#pragma unroll
+        for (int ti = 0; ti < G::TI; ++ti) a[ti] = tr_frag(x, LDI, p0, (wi * G::TI + ti) * 32, lane);
+#pragma unroll
+        for (int tj = 0; tj < G::TJ; ++tj) b[tj] = tr_frag(g, LDO, p0, (wj * G::TJ + tj) * 32, lane);
+#pragma unroll
+        for (int ti = 0; ti < G::TI; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < G::TJ; ++tj)
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ti], b[tj], acc[ti][tj], 0, 0, 0);
+      } else {
+        const int h = lane >> 5, c = lane & 31;
+#pragma unroll
+        for (int m = 0; m < KP / 2; ++m) {
+          float a[G::TI], b[G::TJ];
+#pragma unroll
+          for (int ti = 0; ti < G::TI; ++ti) a[ti] = x[(p0 + 2 * m + h) * LDI + (wi * G::TI + ti) * 32 + c];
+#pragma unroll
+          for (int tj = 0; tj < G::TJ; ++tj) b[tj] = g[(p0 + 2 * m + h) * LDO + (wj * G::TJ + tj) * 32 + c];
+#pragma unroll
+          for (int ti = 0; ti < G::TI; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < G::TJ; ++tj)
+              acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ti], b[tj], acc[ti][tj], 0, 0, 0);
+        }
+      }
+    }
+    if (more) store_rows(cur ^ 1);
+    __syncthreads();
+  }
+
+  // flush: accumulator register r of lane l is row (r/4)*8 + (l/32)*4 + r%4, column l%32
+  const int h = lane >> 5, c = lane & 31;
+#pragma unroll
+  for (int ti = 0; ti < G::TI; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < G::TJ; ++tj) {
+      float *tile = gw32 + ((size_t)k * c_in + ci0 + (wi * G::TI + ti) * 32) * c_out + co0 +
+                    (wj * G::TJ + tj) * 32 + c;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        atomic_add(tile + (size_t)((r / 4) * 8 + h * 4 + (r % 4)) * c_out, acc[ti][tj][r]);
+    }
+}
+
+template <typename T>
+__global__ void add_from_f32_kernel(T *__restrict__ dst, const float *__restrict__ src, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = __float2half(__half2float(dst[i]) + src[i]);
+}
+
+int blocks_of(int c) { return c % 128 == 0 ? 4 : (c % 64 == 0 ? 2 : 1); }
+
+int num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
+      cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+template <typename T, int BI, int BJ>
+int launch(const WgradArgs &a, float *acc32) {
+  using W = WT<T>;
+  constexpr int SP = W::stage_pairs;
+  const int ty = (a.c_in / (32 * BI)) * (a.c_out / (32 * BJ));
+  // enough workgroups to fill the chip a few times over, chunks a multiple of the stage size
+  int64_t want = (int64_t)num_cus() * 4 / ty;
+  if (want < 1) want = 1;
+  int64_t chunk = (a.n_pairs + want - 1) / want;
+  chunk = (chunk + SP - 1) / SP * SP;
+  if (chunk < 4 * SP) chunk = 4 * SP;
+  const int64_t tiles = (a.n_pairs + chunk - 1) / chunk + a.k_vol;
+  const size_t lds = 2 * (size_t)SP * ((BI * 32 + W::pad) + (BJ * 32 + W::pad)) * sizeof(T);
+  auto kern = wgrad_kernel<T, BI, BJ>;
+  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  {
+    ProfileScope prof("wgrad_kernel", a.stream);
+    kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
+        (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
+        a.c_out, (int)chunk);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
+template <typename T>
+int dispatch(const WgradArgs &a, float *acc32) {
+  const int bi = blocks_of(a.c_in), bj = blocks_of(a.c_out);
+#define FGMS_WG(I, J) if (bi == I && bj == J) return launch<T, I, J>(a, acc32);
+  FGMS_WG(1, 1) FGMS_WG(1, 2) FGMS_WG(1, 4)
+  FGMS_WG(2, 1) FGMS_WG(2, 2) FGMS_WG(2, 4)
+  FGMS_WG(4, 1) FGMS_WG(4, 2) FGMS_WG(4, 4)
+#undef FGMS_WG
+  set_error("launch_mfma_wgrad: unsupported shape");
+  return FGMS_E_INVALID;
+}
+
+}  // namespace
+
+bool mfma_wgrad_supported(const WgradArgs &a) {
+  if (a.c_in % 32 != 0 || a.c_out % 32 != 0) return false;
+  if (reinterpret_cast<uintptr_t>(a.in) % 16 || reinterpret_cast<uintptr_t>(a.gout) % 16) return false;
+  return true;
+}
+
+int launch_mfma_wgrad(const WgradArgs &a) {
+  const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+  if (a.dtype == FGMS_F16) {
+    // partial sums of all workgroups meet in fp32 and are rounded to fp16 once
+    void *ws = nullptr;
+    int rc = workspace_get(a.stream, 1, n * sizeof(float), &ws);
+    if (rc != FGMS_OK) return rc;
+    if ((rc = launch_fill_zero(ws, n * sizeof(float), a.stream))) return rc;
+    if ((rc = dispatch<__half>(a, (float *)ws))) return rc;
+    add_from_f32_kernel<__half><<<(unsigned)((n + 255) / 256), 256, 0, a.stream>>>(
+        (__half *)a.gw, (const float *)ws, n);
+    FGMS_HIP_TRY(hipGetLastError());
+    return FGMS_OK;
+  }
+  return dispatch<float>(a, (float *)a.gw);
+}
+
+}  // namespace fgms
