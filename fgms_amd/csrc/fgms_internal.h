@@ -68,6 +68,12 @@ struct Plan {
   int64_t n_in, n_out, n_pairs;
   int32_t *nbr_out;   // [k_vol, n_out]: input row feeding output row o through offset k, or -1
   int32_t *nbr_in;    // [k_vol, n_in]:  output row fed by input row i through offset k, or -1
+  // bit k of mask_out[b] : some row of the 64-row block b has a neighbour through
+  // offset k (only built when k_vol <= 64; the output-stationary kernels need it)
+  unsigned long long *mask_out;  // [ceil(n_out / 64)]
+  unsigned long long *mask_in;   // [ceil(n_in / 64)]
+  unsigned long long *mask32_out; // the same per 32-row block, [2 * ceil(n_out / 64)]
+  unsigned long long *mask32_in;
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -94,5 +100,7 @@ bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_planned_gms(const GmsArgs &a, const Plan *p);
+bool rows2_supported(const GmsArgs &a, const Plan *p);
+int launch_rows2(const GmsArgs &a, const Plan *p);
 
 }  // namespace fgms

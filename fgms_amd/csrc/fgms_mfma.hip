@@ -29,37 +29,15 @@
 
 #include "fgms_device.h"
 #include "fgms_internal.h"
+#include "fgms_mma.h"
 
 namespace fgms {
 namespace {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-typedef float float16v __attribute__((ext_vector_type(16)));
-typedef int int4v __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
 constexpr int kWaveRows = 64;                 // two 32-row MFMA tiles per wave
 constexpr int kTileRows = kWaves * kWaveRows; // 256 rows per workgroup tile
-
-template <typename T> struct Elem;
-template <> struct Elem<__half> { static constexpr int per_chunk = 8; };
-template <> struct Elem<float> { static constexpr int per_chunk = 4; };
-
-template <typename T>
-__device__ __forceinline__ void mma(float16v &acc, const int4v &a, const int4v &b) {
-  if constexpr (sizeof(T) == 2) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a),
-                                                 __builtin_bit_cast(half8, b), acc, 0, 0, 0);
-  } else {
-    const float4v fa = __builtin_bit_cast(float4v, a), fb = __builtin_bit_cast(float4v, b);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1], fb[1], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2], fb[2], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[3], fb[3], acc, 0, 0, 0);
-  }
-}
 
 // LDS ordering between lanes of one wave: LDS operations of a wave complete in
 // program order; the fence keeps the compiler from moving them across.
@@ -167,12 +145,6 @@ __device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__
   }
 }
 
-__device__ __forceinline__ float swap_with_neighbour(float v) {
-  // lane ^ 1 inside each quad: quad_perm [1, 0, 3, 2]
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-}
-
 // Writes a wave's accumulators.  Accumulator register r of lane l holds row
 // (r / 4) * 8 + (l / 32) * 4 + r % 4 and column l % 32 of its 32x32 tile.  For
 // fp16 two lanes swap one value each so that every lane owns two neighbouring
@@ -218,6 +190,62 @@ __device__ __forceinline__ void write_tile(const float16v (&acc)[2][NT], T *__re
         }
       }
     }
+  }
+}
+
+// dst[row0 + r] += acc for the 64 consecutive rows of a wave (no atomics: the
+// caller owns these rows).  All reads of the old values are issued before the
+// first add so that they overlap.
+template <typename T, int NT>
+__device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__restrict__ dst,
+                                         int row0, int n_dst, int c_dst, int cd0, int lane) {
+  const int h = lane / 32, col = lane % 32;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        float old[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
+          old[r] = dst[(size_t)min(row, n_dst - 1) * c_dst + cd0 + nt * 32 + col];
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
+          if (row < n_dst) dst[(size_t)row * c_dst + cd0 + nt * 32 + col] = old[r] + acc[mt][nt][r];
+        }
+      }
+  } else {
+    const bool odd = col & 1;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        __half2 old[8];
+#pragma unroll
+        for (int rp = 0; rp < 8; ++rp) {
+          const int r = 2 * rp + (odd ? 1 : 0);
+          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
+          old[rp] = *reinterpret_cast<const __half2 *>(
+              reinterpret_cast<const __half *>(dst) + (size_t)min(row, n_dst - 1) * c_dst + cd0 +
+              nt * 32 + (col & ~1));
+        }
+#pragma unroll
+        for (int rp = 0; rp < 8; ++rp) {
+          const float v0 = acc[mt][nt][2 * rp], v1 = acc[mt][nt][2 * rp + 1];
+          const float got = swap_with_neighbour(odd ? v0 : v1);
+          const float lo = odd ? got : v0, hi = odd ? v1 : got;
+          const int r = 2 * rp + (odd ? 1 : 0);
+          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
+          const float2 o = __half22float2(old[rp]);
+          if (row < n_dst)
+            *reinterpret_cast<__half2 *>(reinterpret_cast<__half *>(dst) + (size_t)row * c_dst +
+                                         cd0 + nt * 32 + (col & ~1)) =
+                __floats2half2_rn(o.x + lo, o.y + hi);
+        }
+      }
   }
 }
 
@@ -292,41 +320,78 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 // ---------------------------------------------------------------------------
 // Output-stationary kernel.  nbr is the plan's table laid out [k_vol][n_dst]:
 // nbr[k][d] = source row that reaches destination row d through offset k, or -1.
+//
+// The work of a workgroup is a list of stages (offset k, slab of the source
+// row).  Stages are software-pipelined: while the MFMAs of stage t run, the
+// weights and the gathered rows of stage t + 1 are already in flight in
+// registers (the row index of the offset after that is in flight too); they are
+// written to LDS after the MFMAs and one barrier closes the stage.  Weights are
+// double-buffered in LDS, each wave's row tile is single-buffered (only its own
+// wave reads it).
+template <typename T, int S>
+__device__ __forceinline__ void gather_issue(int4v (&v)[2 * S], int (&g)[2 * S],
+                                             const int *__restrict__ idx,
+                                             const T *__restrict__ src, int c_src, int slab,
+                                             int lane) {
+  constexpr int E = Elem<T>::per_chunk;
+  constexpr int C = 2 * S;
+#pragma unroll
+  for (int it = 0; it < C; ++it) g[it] = idx[(it * 64 + lane) / C];
+#pragma unroll
+  for (int it = 0; it < C; ++it) {
+    const int c = (it * 64 + lane) % C;
+    v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(g[it], 0) * c_src +
+                                             (size_t)(slab * C + c) * E);
+  }
+}
+
+template <int S>
+__device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (&v)[2 * S],
+                                              const int (&g)[2 * S], int lane) {
+  constexpr int C = 2 * S;
+#pragma unroll
+  for (int it = 0; it < C; ++it) {
+    const int slot = it * 64 + lane;
+    a_lds[a_slot<S>(slot / C, slot % C)] = g[it] < 0 ? int4v{0, 0, 0, 0} : v[it];
+  }
+}
+
 template <typename T, int NT, int S>
 __global__ __launch_bounds__(kThreads) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
-    const int32_t *__restrict__ nbr, int n_dst, int k_vol, int c_src, int c_dst) {
+    const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
+    int n_dst, int k_vol, int c_src, int c_dst) {
   constexpr int E = Elem<T>::per_chunk;
+  constexpr int C = 2 * S;
+  constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
+  constexpr int NW = (WCH + kThreads - 1) / kThreads;     // ... per thread
   extern __shared__ int4v lds[];
   __shared__ unsigned long long wg_mask;
-  const int slabs = c_src / (2 * S * E);
-  const int qs = slabs * S;
+  const int slabs = c_src / (C * E);
   const int nts = c_dst / 32;
-  int4v *w_lds = lds;
+  int4v *w_lds = lds;                                     // [2][WCH]
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  int4v *a_lds = lds + qs * NT * 64 + wave * (kWaveRows * 2 * S);
-  int *idx_all = reinterpret_cast<int *>(lds + qs * NT * 64 + kWaves * (kWaveRows * 2 * S));
+  int4v *a_lds = lds + 2 * WCH + wave * (kWaveRows * C);
+  int *idx_all = reinterpret_cast<int *>(lds + 2 * WCH + kWaves * (kWaveRows * C));
   int *gidx = idx_all + wave * 2 * kWaveRows;
   int *didx = gidx + kWaveRows;
   const int nt0 = blockIdx.y * NT;
-  const size_t packed_per_k = (size_t)c_src * c_dst / E;
+  const int4v *packed4 = reinterpret_cast<const int4v *>(packed);
+  const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
 
   const int row0 = blockIdx.x * kTileRows + wave * kWaveRows;
   const int my_row = row0 + lane;
   const bool in_range = my_row < n_dst;
   didx[lane] = in_range ? my_row : -1;
 
-  // which offsets touch this wave's rows / this workgroup's rows
-  unsigned long long wave_mask = 0;
-  for (int k = 0; k < k_vol; ++k) {
-    const int g = in_range ? nbr[(size_t)k * n_dst + my_row] : -1;
-    if (__ballot(g >= 0)) wave_mask |= 1ull << k;
-  }
+  // which offsets touch this wave's rows / this workgroup's rows (from the plan)
+  const unsigned long long wave_mask = row0 < n_dst ? block_masks[row0 / 64] : 0ull;
   if (threadIdx.x == 0) wg_mask = 0;
   __syncthreads();
   if (lane == 0 && wave_mask) atomicOr(&wg_mask, wave_mask);
   __syncthreads();
   unsigned long long todo = wg_mask;
+  if (!todo) return;
 
   float16v acc[2][NT];
 #pragma unroll
@@ -336,33 +401,83 @@ __global__ __launch_bounds__(kThreads) void gms_rows_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
 
-  while (todo) {
-    const int k = __builtin_ctzll(todo);
-    todo &= todo - 1;
-    __syncthreads();  // everyone is done with the previous offset's weights
-    load_weights<NT>(w_lds, reinterpret_cast<const int4v *>(packed) + packed_per_k * k, qs, nts, nt0);
-    __syncthreads();
-    if (!((wave_mask >> k) & 1)) continue;
-    const int g = in_range ? nbr[(size_t)k * n_dst + my_row] : -1;
-    gidx[lane] = g;
-    wave_lds_fence();
-    for (int slab = 0; slab < slabs; ++slab) {
-      stage_rows<T, S>(a_lds, gidx, src, c_src, slab, lane);
-      wave_lds_fence();
-      mma_slab<T, NT, S>(acc, a_lds, w_lds, slab, lane);
-      wave_lds_fence();
+  // weights of stage (k, slab): chunks [(slab*S + s) * nts + nt0 + nt] * 64 + lane
+  auto weights_issue = [&](int4v (&wreg)[NW], int k, int slab) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int e = threadIdx.x + kThreads * i;
+      if (NW * kThreads == WCH || e < WCH) {
+        const int q = e / (NT * 64), rem = e % (NT * 64);
+        wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
+      }
     }
-  }
-  if (wave_mask) {
+  };
+  auto weights_commit = [&](const int4v (&wreg)[NW], int buf) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int e = threadIdx.x + kThreads * i;
+      if (NW * kThreads == WCH || e < WCH) w_lds[buf * WCH + e] = wreg[i];
+    }
+  };
+
+  int k = __builtin_ctzll(todo);
+  todo &= todo - 1;
+  int slab = 0;
+  int k_nxt = todo ? __builtin_ctzll(todo) : -1;
+  if (todo) todo &= todo - 1;
+  bool active = (wave_mask >> k) & 1;
+  int4v wreg[NW];
+  int4v v[C];
+  int gsel[C];
+
+  // prologue: stage 0 goes straight to LDS
+  gidx[lane] = in_range ? nbr[(size_t)k * n_dst + my_row] : -1;
+  int g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * n_dst + my_row] : -1;
+  wave_lds_fence();
+  weights_issue(wreg, k, 0);
+  if (active) gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
+  weights_commit(wreg, 0);
+  if (active) gather_commit<S>(a_lds, v, gsel, lane);
+  __syncthreads();
+
+  int buf = 0;
+  while (true) {
+    int nk = k, nslab = slab + 1;
+    if (nslab == slabs) { nk = k_nxt; nslab = 0; }
+    const bool has_next = nk >= 0;
+    const bool next_active = has_next && ((wave_mask >> nk) & 1);
+    if (has_next) {
+      if (nk != k) {          // the row loads that used the old indices were issued a stage ago
+        gidx[lane] = g_nxt;
+        wave_lds_fence();
+      }
+      weights_issue(wreg, nk, nslab);
+      if (next_active) gather_issue<T, S>(v, gsel, gidx, src, c_src, nslab, lane);
+    }
+    if (active) mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+    if (!has_next) break;
     wave_lds_fence();
-    write_tile<T, NT, false>(acc, dst, didx, c_dst, nt0 * 32, lane);
+    if (next_active) gather_commit<S>(a_lds, v, gsel, lane);
+    weights_commit(wreg, buf ^ 1);
+    if (nk != k) {
+      k_nxt = todo ? __builtin_ctzll(todo) : -1;
+      if (todo) todo &= todo - 1;
+      g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * n_dst + my_row] : -1;
+    }
+    __syncthreads();
+    buf ^= 1;
+    k = nk;
+    slab = nslab;
+    active = next_active;
   }
+  if (wave_mask) add_rows<T, NT>(acc, dst, row0, n_dst, c_dst, nt0 * 32, lane);
 }
 
 // ---------------------------------------------------------------------------
 struct Shape {
   int c_src, c_dst, S, NT, E;
-  size_t lds_bytes;
+  size_t lds_bytes;       // pair-stationary kernel
+  size_t lds_rows_bytes;  // output-stationary kernel
   bool ok;
 };
 
@@ -378,9 +493,10 @@ Shape shape_of(const GmsArgs &a) {
   s.NT = (s.c_dst % 64 == 0) ? 2 : 1;
   // rows are read with 16-byte loads and fp16 results written as 4-byte pairs
   if (reinterpret_cast<uintptr_t>(a.src) % 16 || reinterpret_cast<uintptr_t>(a.dst) % 4) return s;
-  s.lds_bytes = (size_t)s.c_src * s.NT * 32 * esz           // weights of one offset
-                + (size_t)kWaves * kWaveRows * 2 * s.S * 16  // staging tiles
-                + (size_t)kWaves * 2 * kWaveRows * sizeof(int);
+  const size_t tiles = (size_t)kWaves * kWaveRows * 2 * s.S * 16  // staging tiles
+                       + (size_t)kWaves * 2 * kWaveRows * sizeof(int);
+  s.lds_bytes = (size_t)s.c_src * s.NT * 32 * esz + tiles;      // + weights of one offset
+  s.lds_rows_bytes = 2 * (size_t)s.S * s.NT * 64 * 16 + tiles;  // + two stages of weights
   s.ok = s.lds_bytes <= 128 * 1024;
   return s;
 }
@@ -400,17 +516,6 @@ int pack_weights(const GmsArgs &a, const Shape &s, const T **packed) {
   return FGMS_OK;
 }
 
-int num_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
-      cus = p.multiProcessorCount;
-    if (cus <= 0) cus = 256;
-  }
-  return cus;
-}
 
 template <typename T, int NT, int S>
 int launch_pairs(const GmsArgs &a, const Shape &s) {
@@ -438,7 +543,8 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
 }
 
 template <typename T, int NT, int S>
-int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr) {
+int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
+                const unsigned long long *masks) {
   const T *packed = nullptr;
   int rc = pack_weights<T>(a, s, &packed);
   if (rc != FGMS_OK) return rc;
@@ -446,11 +552,12 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr) {
   if (gx == 0) return FGMS_OK;
   auto kern = gms_rows_kernel<T, NT, S>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)s.lds_bytes));
+                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)s.lds_rows_bytes));
   {
     ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
-    kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_bytes, a.stream>>>(
-        (const T *)a.src, packed, (T *)a.dst, nbr, (int)a.n_dst, a.k_vol, s.c_src, s.c_dst);
+    kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_rows_bytes, a.stream>>>(
+        (const T *)a.src, packed, (T *)a.dst, nbr, masks, (int)a.n_dst, a.k_vol, s.c_src, s.c_dst);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -469,6 +576,33 @@ int dispatch_shape(const Shape &s, F &&f) {
 }
 
 }  // namespace
+
+int num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
+      cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+int pack_weights_any(const GmsArgs &a, int S, const void **packed) {
+  Shape s{};
+  s.S = S;
+  if (a.dtype == FGMS_F16) {
+    const __half *p = nullptr;
+    int rc = pack_weights<__half>(a, s, &p);
+    *packed = p;
+    return rc;
+  }
+  const float *p = nullptr;
+  int rc = pack_weights<float>(a, s, &p);
+  *packed = p;
+  return rc;
+}
 
 bool mfma_gms_supported(const GmsArgs &a) { return shape_of(a).ok; }
 
@@ -504,12 +638,13 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p) {
     return FGMS_E_INVALID;
   }
   const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
+  const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
   if (a.dtype == FGMS_F16)
     return dispatch_shape<__half>(s, [&](auto nt, auto sv) {
-      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr);
+      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks);
     });
   return dispatch_shape<float>(s, [&](auto nt, auto sv) {
-    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr);
+    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks);
   });
 }
 
