@@ -72,8 +72,6 @@ struct Plan {
   // offset k (only built when k_vol <= 64; the output-stationary kernels need it)
   unsigned long long *mask_out;  // [ceil(n_out / 64)]
   unsigned long long *mask_in;   // [ceil(n_in / 64)]
-  unsigned long long *mask32_out; // the same per 32-row block, [2 * ceil(n_out / 64)]
-  unsigned long long *mask32_in;
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -100,7 +98,5 @@ bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_planned_gms(const GmsArgs &a, const Plan *p);
-bool rows2_supported(const GmsArgs &a, const Plan *p);
-int launch_rows2(const GmsArgs &a, const Plan *p);
 
 }  // namespace fgms

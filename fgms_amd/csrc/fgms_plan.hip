@@ -43,32 +43,23 @@ __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
   if (atomicCAS(&nbr_in[(size_t)k * n_in + i], -1, o) != -1) flags[2] = 1;
 }
 
-// One wave per block of 64 consecutive rows: which offsets have a neighbour
-// there, for the whole block (masks64) and for its two 32-row halves (masks32).
+// One wave per block of 64 consecutive rows: which offsets have a neighbour there.
 __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, int k_vol,
-                                   unsigned long long *__restrict__ masks64,
-                                   unsigned long long *__restrict__ masks32) {
+                                   unsigned long long *__restrict__ masks64) {
   const int block = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
   const int row = block * 64 + (int)(threadIdx.x % 64);
   if (block * 64 >= n_rows) return;
-  unsigned long long lo = 0, hi = 0;
+  unsigned long long m = 0;
   for (int k0 = 0; k0 < k_vol; k0 += 8) {
     int g[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       g[i] = (k0 + i < k_vol && row < n_rows) ? nbr[(size_t)(k0 + i) * n_rows + row] : -1;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const unsigned long long b = __ballot(g[i] >= 0);
-      if (b & 0xffffffffull) lo |= 1ull << (k0 + i);
-      if (b >> 32) hi |= 1ull << (k0 + i);
-    }
+    for (int i = 0; i < 8; ++i)
+      if (__ballot(g[i] >= 0)) m |= 1ull << (k0 + i);
   }
-  if (threadIdx.x % 64 == 0) {
-    masks64[block] = lo | hi;
-    masks32[2 * block] = lo;
-    masks32[2 * block + 1] = hi;   // allocated for an even number of 32-row blocks
-  }
+  if (threadIdx.x % 64 == 0) masks64[block] = m;
 }
 
 int fill_i32(int32_t *p, size_t n, int32_t v, hipStream_t s) {
@@ -104,7 +95,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   hipStream_t s = (hipStream_t)stream;
   Plan *p = new Plan();
   p->k_vol = k_vol; p->n_in = n_in; p->n_out = n_out; p->n_pairs = n_pairs;
-  p->nbr_out = p->nbr_in = nullptr; p->mask_out = p->mask_in = p->mask32_out = p->mask32_in = nullptr;
+  p->nbr_out = p->nbr_in = nullptr; p->mask_out = p->mask_in = nullptr;
   p->fwd_ok = p->dgrad_ok = false;
   int *flags = nullptr;
   int rc = FGMS_OK;
@@ -120,8 +111,6 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       hipMalloc((void **)&p->nbr_in, (si ? si : 1) * sizeof(int32_t)) != hipSuccess ||
       hipMalloc((void **)&p->mask_out, (bo ? bo : 1) * sizeof(unsigned long long)) != hipSuccess ||
       hipMalloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long)) != hipSuccess ||
-      hipMalloc((void **)&p->mask32_out, (bo ? 2 * bo : 2) * sizeof(unsigned long long)) != hipSuccess ||
-      hipMalloc((void **)&p->mask32_in, (bi ? 2 * bi : 2) * sizeof(unsigned long long)) != hipSuccess ||
       hipMalloc((void **)&flags, 4 * sizeof(int)) != hipSuccess) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
@@ -138,8 +127,8 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
     }
   }
   if (k_vol <= 64) {
-    if (bo) block_masks_kernel<<<(unsigned)((bo + 3) / 4), 256, 0, s>>>(p->nbr_out, (int)n_out, k_vol, p->mask_out, p->mask32_out);
-    if (bi) block_masks_kernel<<<(unsigned)((bi + 3) / 4), 256, 0, s>>>(p->nbr_in, (int)n_in, k_vol, p->mask_in, p->mask32_in);
+    if (bo) block_masks_kernel<<<(unsigned)((bo + 3) / 4), 256, 0, s>>>(p->nbr_out, (int)n_out, k_vol, p->mask_out);
+    if (bi) block_masks_kernel<<<(unsigned)((bi + 3) / 4), 256, 0, s>>>(p->nbr_in, (int)n_in, k_vol, p->mask_in);
     if (hipGetLastError() != hipSuccess) {
       set_error("fgms_plan_create: mask build launch failed");
       return fail(FGMS_E_HIP);
@@ -170,8 +159,6 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->nbr_in) (void)hipFree(p->nbr_in);
   if (p->mask_out) (void)hipFree(p->mask_out);
   if (p->mask_in) (void)hipFree(p->mask_in);
-  if (p->mask32_out) (void)hipFree(p->mask32_out);
-  if (p->mask32_in) (void)hipFree(p->mask32_in);
   delete p;
 }
 

@@ -212,6 +212,200 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
     }
 }
 
+// Variant for dW tiles up to 64 x 64: every wave stages its own pairs in its own
+// LDS region and multiplies them into a private copy of the whole tile, so the
+// pair loop has no workgroup barrier at all (the four waves take the chunk's
+// 32-pair stages round-robin); the four partial tiles are summed through LDS
+// once, after the loop.  Each operand fragment read from LDS then feeds two
+// MFMAs instead of one.
+template <typename T> struct WTW;
+template <> struct WTW<__half> { static constexpr int stage_pairs = 32; };
+template <> struct WTW<float> { static constexpr int stage_pairs = 16; };
+
+template <typename T, int BI, int BJ>
+__global__ __launch_bounds__(kThreads) void wgrad_wave_kernel(
+    const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
+    const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk) {
+  using W = WT<T>;
+  constexpr int E = W::E, SP = WTW<T>::stage_pairs, KP = W::step_pairs;
+  constexpr int CI = BI * 32, CO = BJ * 32;
+  constexpr int LDI = CI + W::pad, LDO = CO + W::pad;
+  constexpr int NCI = CI / E, NCO = CO / E;
+  constexpr int NX = SP * NCI / 64, NG = SP * NCO / 64;   // chunks per lane and stage
+  static_assert(NX >= 1 && NG >= 1, "stage too small");
+  extern __shared__ int4v lds[];
+  // Workgroup -> (slice c of the pair list, offset k).  Every offset is cut into
+  // the same number of slices, so slice c of each offset covers about the same
+  // band of rows (pair lists are ordered by row inside an offset).  Workgroups
+  // go to the 8 XCDs round-robin; numbering them so that one XCD gets all the
+  // offsets of a slice lets the rows one offset pulled into that XCD's L2 serve
+  // the other offsets of the slice.
+  const int slices = chunk;               // (slices per offset, a multiple of 8)
+  const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+  const int sl = (idx / k_vol) * 8 + xcd, k = idx % k_vol;
+  if (sl >= slices) return;
+  const int k_first = kpos[k], k_count = kpos[k + 1] - k_first;
+  const int per = (k_count + slices - 1) / slices;
+  const int first = k_first + sl * per;
+  const int count = min(per, k_count - sl * per);
+  if (count <= 0) return;
+  const int tiles_co = c_out / CO;
+  const int ci0 = (blockIdx.y / tiles_co) * CI;
+  const int co0 = (blockIdx.y % tiles_co) * CO;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  T *x = reinterpret_cast<T *>(lds) + (size_t)wave * SP * (LDI + LDO);
+  T *g = x + SP * LDI;
+
+  float16v acc[BI][BJ];
+#pragma unroll
+  for (int a = 0; a < BI; ++a)
+#pragma unroll
+    for (int b = 0; b < BJ; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  const int nstages = (count + SP - 1) / SP;
+  int xi[NX], gi[NG];        // gather rows of the next stage to load
+  int xs[NX], gs[NG];        // ... of the stage in flight (sign = padding row)
+  int4v xr[NX], gr[NG];      // its data
+
+  auto load_idx = [&](int st) {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int p = st * SP + (lane + 64 * i) / NCI;
+      xi[i] = p < count ? imap[first + p] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int p = st * SP + (lane + 64 * i) / NCO;
+      gi[i] = p < count ? omap[first + p] : -1;
+    }
+  };
+  auto load_rows = [&]() {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int cc = (lane + 64 * i) % NCI;
+      xs[i] = xi[i];
+      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)max(xi[i], 0) * c_in + ci0 + cc * E);
+    }
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int cc = (lane + 64 * i) % NCO;
+      gs[i] = gi[i];
+      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)max(gi[i], 0) * c_out + co0 + cc * E);
+    }
+  };
+  auto store_rows = [&]() {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int e = lane + 64 * i;
+      *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
+          xs[i] < 0 ? int4v{0, 0, 0, 0} : xr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int e = lane + 64 * i;
+      *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
+          gs[i] < 0 ? int4v{0, 0, 0, 0} : gr[i];
+    }
+  };
+  auto wave_fence = [] {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  int st = wave;
+  if (st < nstages) {
+    load_idx(st);
+    load_rows();
+    if (st + 4 < nstages) load_idx(st + 4);
+  }
+  while (st < nstages) {
+    store_rows();                   // waits for the stage's rows
+    wave_fence();
+    const int nxt = st + 4;
+    if (nxt < nstages) {
+      load_rows();                  // next stage, in flight during the MFMAs
+      if (nxt + 4 < nstages) load_idx(nxt + 4);
+    }
+#pragma unroll
+    for (int ks = 0; ks < SP / KP; ++ks) {
+      const int p0 = ks * KP;
+      if constexpr (sizeof(T) == 2) {
+        half8 a[BI], b[BJ];
+#pragma unroll
+        for (int ti = 0; ti < BI; ++ti) a[ti] = tr_frag(x, LDI, p0, ti * 32, lane);
+#pragma unroll
+        for (int tj = 0; tj < BJ; ++tj) b[tj] = tr_frag(g, LDO, p0, tj * 32, lane);
+#pragma unroll
+        for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < BJ; ++tj)
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ti], b[tj], acc[ti][tj], 0, 0, 0);
+      } else {
+        const int h = lane >> 5, c = lane & 31;
+#pragma unroll
+        for (int m = 0; m < KP / 2; ++m) {
+          float a[BI], b[BJ];
+#pragma unroll
+          for (int ti = 0; ti < BI; ++ti) a[ti] = x[(p0 + 2 * m + h) * LDI + ti * 32 + c];
+#pragma unroll
+          for (int tj = 0; tj < BJ; ++tj) b[tj] = g[(p0 + 2 * m + h) * LDO + tj * 32 + c];
+#pragma unroll
+          for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < BJ; ++tj)
+              acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ti], b[tj], acc[ti][tj], 0, 0, 0);
+        }
+      }
+    }
+    wave_fence();                   // the tile is rewritten at the top of the loop
+    st = nxt;
+  }
+
+  // sum the four waves' tiles: (2, 3) -> (0, 1), then 1 -> 0, through LDS
+  float *red = reinterpret_cast<float *>(lds);
+  constexpr int kTileFloats = BI * BJ * 16 * 64;
+  auto put = [&](int slot) {
+#pragma unroll
+    for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < BJ; ++tj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          red[(size_t)slot * kTileFloats + ((ti * BJ + tj) * 16 + r) * 64 + lane] = acc[ti][tj][r];
+  };
+  auto take = [&](int slot) {
+#pragma unroll
+    for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < BJ; ++tj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[ti][tj][r] += red[(size_t)slot * kTileFloats + ((ti * BJ + tj) * 16 + r) * 64 + lane];
+  };
+  __syncthreads();
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave != 0) return;
+  take(0);
+  const int h = lane >> 5, c = lane & 31;
+#pragma unroll
+  for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < BJ; ++tj) {
+      float *tile = gw32 + ((size_t)k * c_in + ci0 + ti * 32) * c_out + co0 + tj * 32 + c;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        atomic_add(tile + (size_t)((r / 4) * 8 + h * 4 + (r % 4)) * c_out, acc[ti][tj][r]);
+    }
+}
+
 template <typename T>
 __global__ void add_from_f32_kernel(T *__restrict__ dst, const float *__restrict__ src, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -258,12 +452,44 @@ int launch(const WgradArgs &a, float *acc32) {
   return FGMS_OK;
 }
 
+template <typename T, int BI, int BJ>
+int launch_wave(const WgradArgs &a, float *acc32) {
+  using W = WT<T>;
+  constexpr int SP = WTW<T>::stage_pairs;
+  const int ty = (a.c_in / (32 * BI)) * (a.c_out / (32 * BJ));
+  // slices per offset: enough workgroups to fill the chip a few times, at least
+  // ~16 stages of pairs per slice on average, a multiple of 8 (one per XCD)
+  int64_t slices = (int64_t)num_cus() * 6 / ((int64_t)a.k_vol * ty);
+  const int64_t by_work = a.n_pairs / ((int64_t)a.k_vol * 16 * SP);
+  if (slices > by_work) slices = by_work;
+  slices = (slices + 7) / 8 * 8;
+  if (slices < 8) slices = 8;
+  const int64_t chunk = slices;
+  const int64_t tiles = slices * a.k_vol;
+  size_t lds = 4 * (size_t)SP * ((BI * 32 + W::pad) + (BJ * 32 + W::pad)) * sizeof(T);
+  const size_t red = 2 * (size_t)BI * BJ * 16 * 64 * sizeof(float);
+  if (lds < red) lds = red;
+  auto kern = wgrad_wave_kernel<T, BI, BJ>;
+  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  {
+    ProfileScope prof("wgrad_wave_kernel", a.stream);
+    kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
+        (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
+        a.c_out, (int)chunk);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
 template <typename T>
 int dispatch(const WgradArgs &a, float *acc32) {
   const int bi = blocks_of(a.c_in), bj = blocks_of(a.c_out);
+#define FGMS_WW(I, J) if (bi == I && bj == J) return launch_wave<T, I, J>(a, acc32);
+  FGMS_WW(1, 1) FGMS_WW(1, 2) FGMS_WW(2, 1) FGMS_WW(2, 2)
+#undef FGMS_WW
 #define FGMS_WG(I, J) if (bi == I && bj == J) return launch<T, I, J>(a, acc32);
-  FGMS_WG(1, 1) FGMS_WG(1, 2) FGMS_WG(1, 4)
-  FGMS_WG(2, 1) FGMS_WG(2, 2) FGMS_WG(2, 4)
+  FGMS_WG(1, 4) FGMS_WG(2, 4)
   FGMS_WG(4, 1) FGMS_WG(4, 2) FGMS_WG(4, 4)
 #undef FGMS_WG
   set_error("launch_mfma_wgrad: unsupported shape");

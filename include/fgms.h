@@ -130,9 +130,7 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
 
 /* Selects kernels by hand for tests and profiling: 0 = automatic dispatch,
  * 1 = force the generic (non-MFMA) kernels, 2 = force the pair-stationary MFMA
- * kernels even when a usable plan is passed, 3 = with a plan, force the
- * LDS-staged output-stationary kernel instead of the register-fed one.
- * Process-wide. */
+ * kernels even when a usable plan is passed.  Process-wide. */
 void fgms_set_kernel_policy(int policy);
 
 /*
