@@ -125,6 +125,7 @@ int run_gms(GmsArgs a, const Plan *plan) {
   const bool dense = a.dense_k >= 0;
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
   if (g_policy != 1) {
+    if (!dense && g_policy == 0 && small_gms_supported(a, plan)) return launch_small_gms(a, plan);
     if (!dense && g_policy != 2 && planned_gms_supported(a, plan)) return launch_planned_gms(a, plan);
     if (mfma_gms_supported(a)) return launch_mfma_gms(a);
   }

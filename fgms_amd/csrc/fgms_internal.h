@@ -96,6 +96,8 @@ bool mfma_gms_supported(const GmsArgs &a);
 int launch_mfma_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);
+bool small_gms_supported(const GmsArgs &a, const Plan *p);
+int launch_small_gms(const GmsArgs &a, const Plan *p);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_planned_gms(const GmsArgs &a, const Plan *p);
 

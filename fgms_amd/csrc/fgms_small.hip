@@ -1,0 +1,208 @@
+// Skinny-channel gather-GEMM kernel (no MFMA): layers whose narrow side is at
+// most 16 channels, e.g. the 4 -> 32 first layer of a voxel network.  Such a
+// layer moves ~10x more bytes than it has flops for the matrix cores to matter
+// (a 4-channel fp16 row is 8 bytes), so the kernel is organised around memory:
+//
+//   * output-stationary through the plan's neighbour table: one LANE owns one
+//     destination row and keeps its whole output row in registers, so the
+//     destination is read and written exactly once, 16 bytes at a time, and
+//     there are no atomics;
+//   * the neighbour indices of the 64 rows of a wave are one coalesced 256-byte
+//     line per offset; the gathered source rows are 8..64-byte vector loads;
+//   * all weights (k_vol * c_src * c_dst <= 13824 values) sit in LDS as fp32 and
+//     are read with wave-uniform addresses (LDS broadcast), offsets that no row
+//     of the wave uses are skipped with the plan's 64-row block mask.
+//
+// The reference handles these shapes with its "_once" kernels
+// (backend/spconv.cuh:569-665, 899-992), pair-stationary with scalar atomics.
+#include "fgms_device.h"
+#include "fgms_internal.h"
+
+namespace fgms {
+namespace {
+
+constexpr int kSmallThreads = 256;
+constexpr int kSmallMaxWeights = 13824;   // fp32 values in LDS (54 KB)
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+// N elements starting at p (aligned to min(16, N * sizeof(T)) bytes), widened to fp32.
+template <typename T, int N>
+__device__ __forceinline__ void load_row(float (&x)[N], const T *__restrict__ p) {
+  constexpr int bytes = N * (int)sizeof(T);
+  if constexpr (sizeof(T) == 4) {
+    if constexpr (bytes % 16 == 0) {
+#pragma unroll
+      for (int i = 0; i < N / 4; ++i) {
+        const f32x4 v = reinterpret_cast<const f32x4 *>(p)[i];
+        x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < N / 2; ++i) {
+        const f32x2 v = reinterpret_cast<const f32x2 *>(p)[i];
+        x[2 * i] = v.x; x[2 * i + 1] = v.y;
+      }
+    }
+  } else {
+    if constexpr (bytes % 16 == 0) {
+#pragma unroll
+      for (int i = 0; i < N / 8; ++i) {
+        const f16x8 v = reinterpret_cast<const f16x8 *>(p)[i];
+        x[8 * i] = (float)v.s0; x[8 * i + 1] = (float)v.s1; x[8 * i + 2] = (float)v.s2;
+        x[8 * i + 3] = (float)v.s3; x[8 * i + 4] = (float)v.s4; x[8 * i + 5] = (float)v.s5;
+        x[8 * i + 6] = (float)v.s6; x[8 * i + 7] = (float)v.s7;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < N / 4; ++i) {
+        const f16x4 v = reinterpret_cast<const f16x4 *>(p)[i];
+        x[4 * i] = (float)v.x; x[4 * i + 1] = (float)v.y; x[4 * i + 2] = (float)v.z;
+        x[4 * i + 3] = (float)v.w;
+      }
+    }
+  }
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void add_store_row(T *__restrict__ p, const float (&acc)[N]) {
+  float old[N];
+  load_row<T, N>(old, p);
+  if constexpr (sizeof(T) == 2) {
+    __half2 *q = reinterpret_cast<__half2 *>(p);
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i) q[i] = __floats2half2_rn(old[2 * i] + acc[2 * i], old[2 * i + 1] + acc[2 * i + 1]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; ++i) p[i] = old[i] + acc[i];
+  }
+}
+
+// CS / CD: source / destination channels (compile time: the inner loops unroll
+// fully and the accumulators stay in registers).
+template <typename T, int CS, int CD>
+__global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
+    const T *__restrict__ src, const T *__restrict__ w, T *__restrict__ dst,
+    const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
+    int n_dst, int k_vol, bool transpose_w) {
+  extern __shared__ __align__(16) float w_lds[];   // [k_vol][CS][CD]
+  const int c_in = transpose_w ? CD : CS, c_out = transpose_w ? CS : CD;
+  for (int e = threadIdx.x; e < k_vol * CS * CD; e += kSmallThreads) {
+    const int k = e / (CS * CD), cs = (e / CD) % CS, cd = e % CD;
+    const T *wk = w + (size_t)k * c_in * c_out;
+    w_lds[e] = to_float(transpose_w ? wk[cd * c_out + cs] : wk[cs * c_out + cd]);
+  }
+  __syncthreads();
+  const int row = blockIdx.x * kSmallThreads + threadIdx.x;
+  const int wave_row0 = row & ~63;
+  if (wave_row0 >= n_dst) return;
+  const unsigned long long mask = block_masks[wave_row0 / 64];
+  if (!mask) return;
+  const bool live = row < n_dst;
+  float acc[CD];
+#pragma unroll
+  for (int i = 0; i < CD; ++i) acc[i] = 0.f;
+
+  unsigned long long todo = mask;
+  int k = __builtin_ctzll(todo);
+  todo &= todo - 1;
+  int g = live ? nbr[(size_t)k * n_dst + row] : -1;
+  while (true) {
+    const int kn = todo ? __builtin_ctzll(todo) : -1;
+    if (todo) todo &= todo - 1;
+    const int gn = (kn >= 0 && live) ? nbr[(size_t)kn * n_dst + row] : -1;   // next offset's index in flight
+    if (g >= 0) {
+      float x[CS];
+      load_row<T, CS>(x, src + (size_t)g * CS);
+      const float *wk = w_lds + k * CS * CD;
+#pragma unroll
+      for (int cs = 0; cs < CS; ++cs)
+#pragma unroll
+        for (int cd = 0; cd < CD; ++cd) acc[cd] += x[cs] * wk[cs * CD + cd];
+    }
+    if (kn < 0) break;
+    k = kn;
+    g = gn;
+  }
+  if (live) add_store_row<T, CD>(dst + (size_t)row * CD, acc);
+}
+
+struct Small {
+  int cs, cd;
+  bool ok;
+};
+
+Small small_of(const GmsArgs &a) {
+  Small s{};
+  s.cs = a.transpose_w ? a.c_out : a.c_in;
+  s.cd = a.transpose_w ? a.c_in : a.c_out;
+  const size_t esz = a.dtype == FGMS_F16 ? 2 : 4;
+  auto allowed = [](int c) { return c == 4 || c == 8 || c == 16 || c == 32 || c == 64; };
+  s.ok = allowed(s.cs) && allowed(s.cd) && (s.cs <= 16 || s.cd <= 16) &&
+         (size_t)s.cs * esz % 8 == 0 && (size_t)s.cd * esz % 8 == 0 &&
+         (size_t)a.k_vol * s.cs * s.cd <= kSmallMaxWeights &&
+         reinterpret_cast<uintptr_t>(a.src) % 16 == 0 && reinterpret_cast<uintptr_t>(a.dst) % 16 == 0;
+  return s;
+}
+
+template <typename T, int CS, int CD>
+int launch_small(const GmsArgs &a, const Plan *p) {
+  const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
+  const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
+  const unsigned gx = (unsigned)((a.n_dst + kSmallThreads - 1) / kSmallThreads);
+  if (gx == 0) return FGMS_OK;
+  const size_t lds = (size_t)a.k_vol * CS * CD * sizeof(float);
+  auto kern = gms_small_kernel<T, CS, CD>;
+  {
+    ProfileScope prof(a.transpose_w ? "gms_small_kernel(dgrad)" : "gms_small_kernel(fwd)", a.stream);
+    kern<<<gx, kSmallThreads, lds, a.stream>>>((const T *)a.src, (const T *)a.w, (T *)a.dst, nbr, masks,
+                                               (int)a.n_dst, a.k_vol, a.transpose_w);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
+template <typename T>
+int dispatch_small(const GmsArgs &a, const Small &s, const Plan *p) {
+#define FGMS_SM(S, D) if (s.cs == S && s.cd == D) return launch_small<T, S, D>(a, p);
+  FGMS_SM(4, 4) FGMS_SM(4, 8) FGMS_SM(4, 16) FGMS_SM(4, 32) FGMS_SM(4, 64)
+  FGMS_SM(8, 4) FGMS_SM(8, 8) FGMS_SM(8, 16) FGMS_SM(8, 32) FGMS_SM(8, 64)
+  FGMS_SM(16, 4) FGMS_SM(16, 8) FGMS_SM(16, 16) FGMS_SM(16, 32)
+  FGMS_SM(32, 4) FGMS_SM(32, 8) FGMS_SM(32, 16)
+  FGMS_SM(64, 4) FGMS_SM(64, 8)
+#undef FGMS_SM
+  set_error("launch_small_gms: unsupported shape");
+  return FGMS_E_INVALID;
+}
+
+}  // namespace
+
+bool small_gms_supported(const GmsArgs &a, const Plan *p) {
+  if (!p || a.dense_k >= 0 || a.k_vol > 64 || a.k_vol != p->k_vol) return false;
+  if (a.transpose_w) {
+    if (!p->dgrad_ok || a.n_dst != p->n_in || a.n_src != p->n_out) return false;
+  } else {
+    if (!p->fwd_ok || a.n_dst != p->n_out || a.n_src != p->n_in) return false;
+  }
+  const Small s = small_of(a);
+  if (!s.ok) return false;
+  // shapes listed in dispatch_small
+  if (s.cs == 16 && s.cd == 64) return false;
+  if (s.cs == 64 && s.cd == 16) return false;
+  return true;
+}
+
+int launch_small_gms(const GmsArgs &a, const Plan *p) {
+  const Small s = small_of(a);
+  if (!small_gms_supported(a, p)) {
+    set_error("launch_small_gms: unsupported shape or plan");
+    return FGMS_E_INVALID;
+  }
+  if (a.dtype == FGMS_F16) return dispatch_small<__half>(a, s, p);
+  return dispatch_small<float>(a, s, p);
+}
+
+}  // namespace fgms
