@@ -105,6 +105,8 @@ def main():
     ap.add_argument("--no-plan", action="store_true", help="do not pass a kernel-map plan")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--scale", type=float, default=1.0, help="voxel-count scale (1.0 = the named size)")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run plain 256 MiB device copies (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (every figure is "
@@ -137,6 +139,13 @@ def main():
         if "wgrad" in passes:
             capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
 
+    if args.copy_calib:
+        a_ = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        b_ = torch.empty_like(a_)
+        for _ in range(3):
+            b_.copy_(a_)
+        torch.cuda.synchronize()
+        del a_, b_
     for _ in range(args.warmup):
         step()
     out.zero_(); gi.zero_(); gw.zero_()
