@@ -43,7 +43,16 @@ std::mutex g_ws_mutex;
 std::map<WsKey, WsBuf> g_ws;
 }  // namespace
 
-int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr) {
+size_t workspace_bytes(hipStream_t stream, int slot) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_ws.find(WsKey{dev, stream, slot});
+  return it == g_ws.end() ? 0 : it->second.bytes;
+}
+
+int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *fresh) {
+  if (fresh) *fresh = false;
   int dev = 0;
   FGMS_HIP_TRY(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(g_ws_mutex);
@@ -63,6 +72,7 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr) {
       return FGMS_E_NOMEM;
     }
     b.bytes = want;
+    if (fresh) *fresh = true;
   }
   *ptr = b.ptr;
   return FGMS_OK;

@@ -208,7 +208,7 @@ int launch_generic_wgrad(const WgradArgs &a) {
   if (a.dtype == FGMS_F16) {
     // accumulate in fp32 and round once; fp16 atomics would round per chunk
     void *ws = nullptr;
-    int rc = workspace_get(a.stream, 1, n * sizeof(float), &ws);
+    int rc = workspace_get(a.stream, 2, n * sizeof(float), &ws);
     if (rc != FGMS_OK) return rc;
     acc32 = (float *)ws;
     rc = launch_fill_zero(acc32, n * sizeof(float), a.stream);

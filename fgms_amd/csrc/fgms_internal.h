@@ -66,8 +66,14 @@ struct Plan {
   int device;
   int k_vol;
   int64_t n_in, n_out, n_pairs;
-  int32_t *nbr_out;   // [k_vol, n_out]: input row feeding output row o through offset k, or -1
-  int32_t *nbr_in;    // [k_vol, n_in]:  output row fed by input row i through offset k, or -1
+  // Destination rows are visited in a plan-chosen order (rows with the same set
+  // of offsets next to each other, inside windows of 4096 rows): position p of
+  // the order is row perm[p] (perm == nullptr: identity).  The tables and masks
+  // below are indexed by POSITION.
+  int32_t *perm_out;  // [n_out]
+  int32_t *perm_in;   // [n_in]
+  int32_t *nbr_out;   // [k_vol, n_out]: input row feeding the output row at position p through offset k, or -1
+  int32_t *nbr_in;    // [k_vol, n_in]:  output row fed by the input row at position p through offset k, or -1
   // bit k of mask_out[b] : some row of the 64-row block b has a neighbour through
   // offset k (only built when k_vol <= 64; the output-stationary kernels need it)
   unsigned long long *mask_out;  // [ceil(n_out / 64)]
@@ -77,8 +83,11 @@ struct Plan {
 };
 
 // Fp32 scratch that outlives a call (per device and stream, grown on demand).
-// slot 0: packed weights, slot 1: fp32 weight-gradient accumulator.
-int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr);
+// slot 0: packed weights, slot 1: fp32 weight-gradient accumulator of the MFMA kernels (kept
+// all-zero between calls), slot 2: the generic kernel's accumulator.
+// *fresh (optional) is set when the buffer was (re)allocated by this call.
+int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *fresh = nullptr);
+size_t workspace_bytes(hipStream_t stream, int slot);
 
 // Brackets a main-kernel launch with events when profiling is enabled.
 struct ProfileScope {

@@ -193,59 +193,62 @@ __device__ __forceinline__ void write_tile(const float16v (&acc)[2][NT], T *__re
   }
 }
 
-// dst[row0 + r] += acc for the 64 consecutive rows of a wave (no atomics: the
-// caller owns these rows).  All reads of the old values are issued before the
-// first add so that they overlap.
+// dst[rows[r]] += acc for the 64 rows of a wave (rows[] in LDS, -1 = none; no
+// atomics: the caller owns these rows).  All reads of the old values are issued
+// before the first add so that they overlap.
 template <typename T, int NT>
 __device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__restrict__ dst,
-                                         int row0, int n_dst, int c_dst, int cd0, int lane) {
+                                         const int *__restrict__ rows, int c_dst, int cd0,
+                                         int lane) {
   const int h = lane / 32, col = lane % 32;
   if constexpr (sizeof(T) == 4) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < 2; ++mt) {
+      int row[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) row[r] = rows[mt * 32 + (r / 4) * 8 + h * 4 + (r % 4)];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         float old[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
-          old[r] = dst[(size_t)min(row, n_dst - 1) * c_dst + cd0 + nt * 32 + col];
-        }
+        for (int r = 0; r < 16; ++r)
+          old[r] = dst[(size_t)max(row[r], 0) * c_dst + cd0 + nt * 32 + col];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
-          if (row < n_dst) dst[(size_t)row * c_dst + cd0 + nt * 32 + col] = old[r] + acc[mt][nt][r];
-        }
+        for (int r = 0; r < 16; ++r)
+          if (row[r] >= 0) dst[(size_t)row[r] * c_dst + cd0 + nt * 32 + col] = old[r] + acc[mt][nt][r];
       }
+    }
   } else {
     const bool odd = col & 1;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < 2; ++mt) {
+      int row[8];
+#pragma unroll
+      for (int rp = 0; rp < 8; ++rp) {
+        const int r = 2 * rp + (odd ? 1 : 0);
+        row[rp] = rows[mt * 32 + (r / 4) * 8 + h * 4 + (r % 4)];
+      }
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         __half2 old[8];
 #pragma unroll
-        for (int rp = 0; rp < 8; ++rp) {
-          const int r = 2 * rp + (odd ? 1 : 0);
-          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
+        for (int rp = 0; rp < 8; ++rp)
           old[rp] = *reinterpret_cast<const __half2 *>(
-              reinterpret_cast<const __half *>(dst) + (size_t)min(row, n_dst - 1) * c_dst + cd0 +
+              reinterpret_cast<const __half *>(dst) + (size_t)max(row[rp], 0) * c_dst + cd0 +
               nt * 32 + (col & ~1));
-        }
 #pragma unroll
         for (int rp = 0; rp < 8; ++rp) {
           const float v0 = acc[mt][nt][2 * rp], v1 = acc[mt][nt][2 * rp + 1];
           const float got = swap_with_neighbour(odd ? v0 : v1);
           const float lo = odd ? got : v0, hi = odd ? v1 : got;
-          const int r = 2 * rp + (odd ? 1 : 0);
-          const int row = row0 + mt * 32 + (r / 4) * 8 + h * 4 + (r % 4);
           const float2 o = __half22float2(old[rp]);
-          if (row < n_dst)
-            *reinterpret_cast<__half2 *>(reinterpret_cast<__half *>(dst) + (size_t)row * c_dst +
+          if (row[rp] >= 0)
+            *reinterpret_cast<__half2 *>(reinterpret_cast<__half *>(dst) + (size_t)row[rp] * c_dst +
                                          cd0 + nt * 32 + (col & ~1)) =
                 __floats2half2_rn(o.x + lo, o.y + hi);
         }
       }
+    }
   }
 }
 
@@ -360,7 +363,7 @@ template <typename T, int NT, int S>
 __global__ __launch_bounds__(kThreads) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
-    int n_dst, int k_vol, int c_src, int c_dst) {
+    const int32_t *__restrict__ perm, int n_dst, int k_vol, int c_src, int c_dst) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
   constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
@@ -382,7 +385,7 @@ __global__ __launch_bounds__(kThreads) void gms_rows_kernel(
   const int row0 = blockIdx.x * kTileRows + wave * kWaveRows;
   const int my_row = row0 + lane;
   const bool in_range = my_row < n_dst;
-  didx[lane] = in_range ? my_row : -1;
+  didx[lane] = in_range ? (perm ? perm[my_row] : my_row) : -1;   // my_row is a position in the plan's row order
 
   // which offsets touch this wave's rows / this workgroup's rows (from the plan)
   const unsigned long long wave_mask = row0 < n_dst ? block_masks[row0 / 64] : 0ull;
@@ -470,7 +473,10 @@ __global__ __launch_bounds__(kThreads) void gms_rows_kernel(
     slab = nslab;
     active = next_active;
   }
-  if (wave_mask) add_rows<T, NT>(acc, dst, row0, n_dst, c_dst, nt0 * 32, lane);
+  if (wave_mask) {
+    wave_lds_fence();
+    add_rows<T, NT>(acc, dst, didx, c_dst, nt0 * 32, lane);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -544,7 +550,7 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
 
 template <typename T, int NT, int S>
 int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
-                const unsigned long long *masks) {
+                const unsigned long long *masks, const int32_t *perm) {
   const T *packed = nullptr;
   int rc = pack_weights<T>(a, s, &packed);
   if (rc != FGMS_OK) return rc;
@@ -557,7 +563,8 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   {
     ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
     kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_rows_bytes, a.stream>>>(
-        (const T *)a.src, packed, (T *)a.dst, nbr, masks, (int)a.n_dst, a.k_vol, s.c_src, s.c_dst);
+        (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, (int)a.n_dst, a.k_vol, s.c_src,
+        s.c_dst);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -639,12 +646,13 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p) {
   }
   const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
   const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
+  const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
   if (a.dtype == FGMS_F16)
     return dispatch_shape<__half>(s, [&](auto nt, auto sv) {
-      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks);
+      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm);
     });
   return dispatch_shape<float>(s, [&](auto nt, auto sv) {
-    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks);
+    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm);
   });
 }
 

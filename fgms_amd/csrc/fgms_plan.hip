@@ -5,6 +5,8 @@
 // rows for one offset as one 256-byte line.  The reference keeps only the pair lists and scatters with atomics
 // (backend/spconv.cuh:457-563); the tables let a workgroup own a block of
 // output rows and sum all offsets in registers.
+#include <stdlib.h>
+
 #include "fgms_device.h"
 #include "fgms_internal.h"
 
@@ -62,6 +64,63 @@ __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, 
   if (threadIdx.x % 64 == 0) masks64[block] = m;
 }
 
+// rmask[row] = bit k set iff row has a neighbour through offset k.
+__global__ void row_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, int k_vol,
+                                 unsigned long long *__restrict__ rmask) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= n_rows) return;
+  unsigned long long m = 0;
+  for (int k = 0; k < k_vol; ++k)
+    if (nbr[(size_t)k * n_rows + row] >= 0) m |= 1ull << k;
+  rmask[row] = m;
+}
+
+// Row order inside windows of kSortWindow consecutive rows: rows are sorted by
+// their offset mask (ties by row number), so that the 64 rows a wave works on
+// use nearly the same offsets and whole (block, offset) steps can be skipped,
+// while a window stays a compact, cache-friendly range of the tensors.  One
+// workgroup bitonic-sorts one window in LDS.
+constexpr int kSortWindow = 4096;
+__global__ __launch_bounds__(1024) void window_sort_kernel(
+    const unsigned long long *__restrict__ rmask, int n_rows, int32_t *__restrict__ perm) {
+  __shared__ unsigned long long key[kSortWindow];
+  __shared__ unsigned short idx[kSortWindow];
+  const int base = blockIdx.x * kSortWindow;
+  for (int i = threadIdx.x; i < kSortWindow; i += blockDim.x) {
+    key[i] = base + i < n_rows ? rmask[base + i] : ~0ull;   // padding sorts to the end
+    idx[i] = (unsigned short)i;
+  }
+  __syncthreads();
+  for (int size = 2; size <= kSortWindow; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int t = threadIdx.x; t < kSortWindow / 2; t += blockDim.x) {
+        const int lo = 2 * t - (t & (stride - 1));
+        const int hi = lo + stride;
+        const bool up = (lo & size) == 0;
+        const unsigned long long ka = key[lo], kb = key[hi];
+        const unsigned short ia = idx[lo], ib = idx[hi];
+        const bool a_after_b = ka > kb || (ka == kb && ia > ib);
+        if (a_after_b == up) {
+          key[lo] = kb; key[hi] = ka;
+          idx[lo] = ib; idx[hi] = ia;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = threadIdx.x; i < kSortWindow; i += blockDim.x)
+    if (base + i < n_rows) perm[base + i] = base + idx[i];
+}
+
+// out[k][pos] = in[k][perm[pos]]
+__global__ void permute_table_kernel(const int32_t *__restrict__ in, const int32_t *__restrict__ perm,
+                                     int n_rows, int k_vol, int32_t *__restrict__ out) {
+  const int pos = blockIdx.x * blockDim.x + threadIdx.x;
+  if (pos >= n_rows) return;
+  const int row = perm[pos];
+  for (int k = 0; k < k_vol; ++k) out[(size_t)k * n_rows + pos] = in[(size_t)k * n_rows + row];
+}
+
 int fill_i32(int32_t *p, size_t n, int32_t v, hipStream_t s) {
   if (n == 0) return FGMS_OK;
   size_t blocks = (n + 1023) / 1024;
@@ -96,6 +155,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   Plan *p = new Plan();
   p->k_vol = k_vol; p->n_in = n_in; p->n_out = n_out; p->n_pairs = n_pairs;
   p->nbr_out = p->nbr_in = nullptr; p->mask_out = p->mask_in = nullptr;
+  p->perm_out = p->perm_in = nullptr;
   p->fwd_ok = p->dgrad_ok = false;
   int *flags = nullptr;
   int rc = FGMS_OK;
@@ -126,20 +186,60 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
+  // Reorder the rows (window sort by offset mask), then derive the block masks
+  // from the tables in their final order.  Temporaries are freed after the
+  // stream synchronisation below.
+  int32_t *tmp_tab[2] = {nullptr, nullptr};
+  unsigned long long *tmp_mask[2] = {nullptr, nullptr};
+  auto free_tmp = [&]() {
+    for (int d = 0; d < 2; ++d) {
+      if (tmp_tab[d]) (void)hipFree(tmp_tab[d]);
+      if (tmp_mask[d]) (void)hipFree(tmp_mask[d]);
+      tmp_tab[d] = nullptr; tmp_mask[d] = nullptr;
+    }
+  };
+  static const bool sort_rows = !(getenv("FGMS_PLAN_SORT") && atoi(getenv("FGMS_PLAN_SORT")) == 0);
   if (k_vol <= 64) {
-    if (bo) block_masks_kernel<<<(unsigned)((bo + 3) / 4), 256, 0, s>>>(p->nbr_out, (int)n_out, k_vol, p->mask_out);
-    if (bi) block_masks_kernel<<<(unsigned)((bi + 3) / 4), 256, 0, s>>>(p->nbr_in, (int)n_in, k_vol, p->mask_in);
+    for (int d = 0; d < 2; ++d) {
+      const int64_t n = d ? n_in : n_out;
+      const size_t blocks = d ? bi : bo;
+      int32_t *&tab = d ? p->nbr_in : p->nbr_out;
+      int32_t *&perm = d ? p->perm_in : p->perm_out;
+      unsigned long long *mask = d ? p->mask_in : p->mask_out;
+      if (n == 0) continue;
+      if (sort_rows && n > 64) {
+        int32_t *sorted = nullptr;
+        if (hipMalloc((void **)&tmp_mask[d], (size_t)n * sizeof(unsigned long long)) != hipSuccess ||
+            hipMalloc((void **)&perm, (size_t)n * sizeof(int32_t)) != hipSuccess ||
+            hipMalloc((void **)&sorted, (size_t)n * k_vol * sizeof(int32_t)) != hipSuccess) {
+          if (sorted) (void)hipFree(sorted);
+          free_tmp();
+          set_error("fgms_plan_create: reorder allocation failed");
+          return fail(FGMS_E_NOMEM);
+        }
+        row_masks_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(tab, (int)n, k_vol, tmp_mask[d]);
+        window_sort_kernel<<<(unsigned)((n + kSortWindow - 1) / kSortWindow), 1024, 0, s>>>(
+            tmp_mask[d], (int)n, perm);
+        permute_table_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(tab, perm, (int)n, k_vol, sorted);
+        tmp_tab[d] = tab;      // the unsorted table, freed after the sync
+        tab = sorted;
+      }
+      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask);
+    }
     if (hipGetLastError() != hipSuccess) {
-      set_error("fgms_plan_create: mask build launch failed");
+      free_tmp();
+      set_error("fgms_plan_create: reorder / mask build launch failed");
       return fail(FGMS_E_HIP);
     }
   }
   int h[4] = {0, 0, 0, 0};
   if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
       hipStreamSynchronize(s) != hipSuccess) {
+    free_tmp();
     set_error("fgms_plan_create: reading the build flags failed");
     return fail(FGMS_E_HIP);
   }
+  free_tmp();
   (void)hipFree(flags);
   flags = nullptr;
   if (h[0]) {
@@ -159,6 +259,8 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->nbr_in) (void)hipFree(p->nbr_in);
   if (p->mask_out) (void)hipFree(p->mask_out);
   if (p->mask_in) (void)hipFree(p->mask_in);
+  if (p->perm_out) (void)hipFree(p->perm_out);
+  if (p->perm_in) (void)hipFree(p->perm_in);
   delete p;
 }
 

@@ -87,7 +87,7 @@ template <typename T, int CS, int CD>
 __global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
     const T *__restrict__ src, const T *__restrict__ w, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
-    int n_dst, int k_vol, bool transpose_w) {
+    const int32_t *__restrict__ perm, int n_dst, int k_vol, bool transpose_w) {
   extern __shared__ __align__(16) float w_lds[];   // [k_vol][CS][CD]
   const int c_in = transpose_w ? CD : CS, c_out = transpose_w ? CS : CD;
   for (int e = threadIdx.x; e < k_vol * CS * CD; e += kSmallThreads) {
@@ -127,7 +127,8 @@ __global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
     k = kn;
     g = gn;
   }
-  if (live) add_store_row<T, CD>(dst + (size_t)row * CD, acc);
+  // `row` is a position in the plan's row order
+  if (live) add_store_row<T, CD>(dst + (size_t)(perm ? perm[row] : row) * CD, acc);
 }
 
 struct Small {
@@ -152,6 +153,7 @@ template <typename T, int CS, int CD>
 int launch_small(const GmsArgs &a, const Plan *p) {
   const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
   const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
+  const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
   const unsigned gx = (unsigned)((a.n_dst + kSmallThreads - 1) / kSmallThreads);
   if (gx == 0) return FGMS_OK;
   const size_t lds = (size_t)a.k_vol * CS * CD * sizeof(float);
@@ -159,7 +161,7 @@ int launch_small(const GmsArgs &a, const Plan *p) {
   {
     ProfileScope prof(a.transpose_w ? "gms_small_kernel(dgrad)" : "gms_small_kernel(fwd)", a.stream);
     kern<<<gx, kSmallThreads, lds, a.stream>>>((const T *)a.src, (const T *)a.w, (T *)a.dst, nbr, masks,
-                                               (int)a.n_dst, a.k_vol, a.transpose_w);
+                                               perm, (int)a.n_dst, a.k_vol, a.transpose_w);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;

@@ -406,10 +406,15 @@ __global__ __launch_bounds__(kThreads) void wgrad_wave_kernel(
     }
 }
 
+// dst[i] += acc[i] rounded once to fp16, and acc[i] is reset: the accumulator is
+// handed back all-zero, which is the state the next call expects to find it in.
 template <typename T>
-__global__ void add_from_f32_kernel(T *__restrict__ dst, const float *__restrict__ src, size_t n) {
+__global__ void add_and_clear_kernel(T *__restrict__ dst, float *__restrict__ acc, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) dst[i] = __float2half(__half2float(dst[i]) + src[i]);
+  if (i < n) {
+    dst[i] = __float2half(__half2float(dst[i]) + acc[i]);
+    acc[i] = 0.f;
+  }
 }
 
 int blocks_of(int c) { return c % 128 == 0 ? 4 : (c % 64 == 0 ? 2 : 1); }
@@ -507,14 +512,20 @@ bool mfma_wgrad_supported(const WgradArgs &a) {
 int launch_mfma_wgrad(const WgradArgs &a) {
   const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
   if (a.dtype == FGMS_F16) {
-    // partial sums of all workgroups meet in fp32 and are rounded to fp16 once
+    // partial sums of all workgroups meet in fp32 and are rounded to fp16 once.
+    // The accumulator is zero-filled when it is (re)allocated and left zero by
+    // every call, so no fill launch is needed per call.
     void *ws = nullptr;
-    int rc = workspace_get(a.stream, 1, n * sizeof(float), &ws);
+    bool fresh = false;
+    int rc = workspace_get(a.stream, 1, n * sizeof(float), &ws, &fresh);
     if (rc != FGMS_OK) return rc;
-    if ((rc = launch_fill_zero(ws, n * sizeof(float), a.stream))) return rc;
-    if ((rc = dispatch<__half>(a, (float *)ws))) return rc;
-    add_from_f32_kernel<__half><<<(unsigned)((n + 255) / 256), 256, 0, a.stream>>>(
-        (__half *)a.gw, (const float *)ws, n);
+    if (fresh && (rc = launch_fill_zero(ws, workspace_bytes(a.stream, 1), a.stream))) return rc;
+    if ((rc = dispatch<__half>(a, (float *)ws))) {
+      (void)launch_fill_zero(ws, workspace_bytes(a.stream, 1), a.stream);
+      return rc;
+    }
+    add_and_clear_kernel<__half><<<(unsigned)((n + 255) / 256), 256, 0, a.stream>>>(
+        (__half *)a.gw, (float *)ws, n);
     FGMS_HIP_TRY(hipGetLastError());
     return FGMS_OK;
   }
