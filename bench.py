@@ -60,39 +60,57 @@ def dataflow_bytes(L, which):
     return m * (L["c_in"] + L["c_out"]) * s + 8 * m + L["k_vol"] * L["c_in"] * L["c_out"] * s
 
 
-def cpu_baseline(name, budget_s=15.0):
+def cpu_baseline(name, budget_s=12.0):
     """Times the CPU oracle (OpenMP, this box's host cores) on a bounded sample of
     the same workload and returns effective TFLOP/s."""
     from oracle import fgms_oracle as oracle
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
     threads = max(1, min(threads, oracle.max_threads() if oracle.max_threads() > 0 else threads))
 
-    def run(scale):
+    def run(scale, repeats=1):
         L, passes, _ = make_case(name, scale)
         args = (L["knnz"], L["imap"], L["omap"])
         t0 = time.perf_counter()
-        if "fwd" in passes:
-            oracle.c_fwd(L["in_feats"], L["kernel"], *args, L["n_out"], threads=threads)
-        if "dgrad" in passes:
-            oracle.c_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"], threads=threads)
-        if "wgrad" in passes:
-            oracle.c_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"], threads=threads)
+        for _ in range(repeats):
+            if "fwd" in passes:
+                oracle.c_fwd(L["in_feats"], L["kernel"], *args, L["n_out"], threads=threads)
+            if "dgrad" in passes:
+                oracle.c_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"], threads=threads)
+            if "wgrad" in passes:
+                oracle.c_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"], threads=threads)
         dt = time.perf_counter() - t0
-        flops = len(passes) * 2.0 * len(L["imap"]) * L["c_in"] * L["c_out"]
+        flops = repeats * len(passes) * 2.0 * len(L["imap"]) * L["c_in"] * L["c_out"]
         return dt, flops, L
 
     scale = 0.05
     dt, flops, L = run(scale)          # probe, then a sample sized to the budget
     want = min(1.0, scale * budget_s / max(dt, 1e-3))
+    repeats = 1
     if want > 1.2 * scale:
+        # the full cloud costs dt / scale per repeat; repeat it to fill the budget
+        repeats = max(1, min(200, int(budget_s / max(dt / scale * want, 1e-3))))
         scale = want
-        dt, flops, L = run(scale)
+        dt, flops, L = run(scale, repeats)
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": "%s at %.0f%% of the voxels (%d voxels, %d pairs), one pass each of %s, %.1f s"
-                  % (name.split("-")[0] + " cloud", scale * 100, L["n_in"], len(L["imap"]),
+        "sample": "%s at %.0f%% of the voxels (%d voxels, %d pairs), %d x one pass each of %s, %.1f s"
+                  % (name.split("-")[0] + " cloud", scale * 100, L["n_in"], len(L["imap"]), repeats,
                      "+".join(WORKLOADS[name][2]), dt),
     }
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` on `workload`, from the committed
+    rocprofv3 FETCH_SIZE / WRITE_SIZE summary (profiles/hbm_traffic.json: KiB per
+    dispatch and the factors a plain copy of known size calibrates them with).
+    None when that workload / kernel was not profiled."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            t = json.load(f)
+        e = t["workloads"][workload][kernel.split("(")[0]]
+        return (e["fetch_kib"] * t["fetch_factor"] + e["write_kib"] * t["write_factor"]) * 1024.0
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main():
@@ -179,12 +197,12 @@ def main():
             which = "dgrad" if "dgrad" in dom else "fwd"
             ach = dataflow_bytes(L, which) / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": PEAK_HBM_GBS,
-                        "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
+                        "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": measured_traffic(args.workload, dom),
                         "avg_kernel_ms": kernels[dom]["avg_ms"]}
         else:
             ach = flops_pass / avg_s / 1e12
             roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_TFLOPS[arith],
-                        "unit": "TFLOP/s", "frac": ach / PEAK_TFLOPS[arith], "traffic": None,
+                        "unit": "TFLOP/s", "frac": ach / PEAK_TFLOPS[arith], "traffic": measured_traffic(args.workload, dom),
                         "avg_kernel_ms": kernels[dom]["avg_ms"]}
 
     line = {
