@@ -67,7 +67,7 @@ struct Plan {
   int k_vol;
   int64_t n_in, n_out, n_pairs;
   // Destination rows are visited in a plan-chosen order (rows with the same set
-  // of offsets next to each other, inside windows of 4096 rows): position p of
+  // of offsets next to each other: a stable sort by offset mask): position p of
   // the order is row perm[p] (perm == nullptr: identity).  The tables and masks
   // below are indexed by POSITION.
   int32_t *perm_out;  // [n_out]

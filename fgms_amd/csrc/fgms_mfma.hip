@@ -360,7 +360,7 @@ __device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (
 }
 
 template <typename T, int NT, int S>
-__global__ __launch_bounds__(kThreads) void gms_rows_kernel(
+__global__ __launch_bounds__(kThreads, 3) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, int n_dst, int k_vol, int c_src, int c_dst) {

@@ -6,6 +6,11 @@
 // (backend/spconv.cuh:457-563); the tables let a workgroup own a block of
 // output rows and sum all offsets in registers.
 #include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+#include <rocprim/device/device_radix_sort.hpp>
 
 #include "fgms_device.h"
 #include "fgms_internal.h"
@@ -75,41 +80,14 @@ __global__ void row_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, in
   rmask[row] = m;
 }
 
-// Row order inside windows of kSortWindow consecutive rows: rows are sorted by
-// their offset mask (ties by row number), so that the 64 rows a wave works on
-// use nearly the same offsets and whole (block, offset) steps can be skipped,
-// while a window stays a compact, cache-friendly range of the tensors.  One
-// workgroup bitonic-sorts one window in LDS.
-constexpr int kSortWindow = 4096;
-__global__ __launch_bounds__(1024) void window_sort_kernel(
-    const unsigned long long *__restrict__ rmask, int n_rows, int32_t *__restrict__ perm) {
-  __shared__ unsigned long long key[kSortWindow];
-  __shared__ unsigned short idx[kSortWindow];
-  const int base = blockIdx.x * kSortWindow;
-  for (int i = threadIdx.x; i < kSortWindow; i += blockDim.x) {
-    key[i] = base + i < n_rows ? rmask[base + i] : ~0ull;   // padding sorts to the end
-    idx[i] = (unsigned short)i;
-  }
-  __syncthreads();
-  for (int size = 2; size <= kSortWindow; size <<= 1) {
-    for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int t = threadIdx.x; t < kSortWindow / 2; t += blockDim.x) {
-        const int lo = 2 * t - (t & (stride - 1));
-        const int hi = lo + stride;
-        const bool up = (lo & size) == 0;
-        const unsigned long long ka = key[lo], kb = key[hi];
-        const unsigned short ia = idx[lo], ib = idx[hi];
-        const bool a_after_b = ka > kb || (ka == kb && ia > ib);
-        if (a_after_b == up) {
-          key[lo] = kb; key[hi] = ka;
-          idx[lo] = ib; idx[hi] = ia;
-        }
-      }
-      __syncthreads();
-    }
-  }
-  for (int i = threadIdx.x; i < kSortWindow; i += blockDim.x)
-    if (base + i < n_rows) perm[base + i] = base + idx[i];
+// Row order: rows are sorted by their offset mask (stable, so rows with equal
+// masks keep their relative order and with it most of their spatial locality).
+// The 64 rows a wave works on then use nearly the same offsets and whole
+// (block, offset) steps can be skipped: on a surface-like cloud of 200 k voxels
+// the number of such steps drops from 68.6 k to 36.7 k (33 k would be perfect).
+__global__ void iota_kernel(int32_t *__restrict__ p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = i;
 }
 
 // out[k][pos] = in[k][perm[pos]]
@@ -186,17 +164,20 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
-  // Reorder the rows (window sort by offset mask), then derive the block masks
+  // Reorder the rows (stable sort by offset mask), then derive the block masks
   // from the tables in their final order.  Temporaries are freed after the
   // stream synchronisation below.
   int32_t *tmp_tab[2] = {nullptr, nullptr};
   unsigned long long *tmp_mask[2] = {nullptr, nullptr};
+  std::vector<void *> tmp_more;
   auto free_tmp = [&]() {
     for (int d = 0; d < 2; ++d) {
       if (tmp_tab[d]) (void)hipFree(tmp_tab[d]);
       if (tmp_mask[d]) (void)hipFree(tmp_mask[d]);
       tmp_tab[d] = nullptr; tmp_mask[d] = nullptr;
     }
+    for (void *q : tmp_more) (void)hipFree(q);
+    tmp_more.clear();
   };
   static const bool sort_rows = !(getenv("FGMS_PLAN_SORT") && atoi(getenv("FGMS_PLAN_SORT")) == 0);
   if (k_vol <= 64) {
@@ -218,8 +199,30 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
           return fail(FGMS_E_NOMEM);
         }
         row_masks_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(tab, (int)n, k_vol, tmp_mask[d]);
-        window_sort_kernel<<<(unsigned)((n + kSortWindow - 1) / kSortWindow), 1024, 0, s>>>(
-            tmp_mask[d], (int)n, perm);
+        // stable LSD radix sort over the k_vol significant bits of the masks
+        unsigned long long *keys_out = nullptr;
+        int32_t *rows_in = nullptr;
+        void *sort_tmp = nullptr;
+        size_t sort_bytes = 0;
+        bool ok = hipMalloc((void **)&keys_out, (size_t)n * sizeof(unsigned long long)) == hipSuccess;
+        if (ok) tmp_more.push_back(keys_out);
+        ok = ok && hipMalloc((void **)&rows_in, (size_t)n * sizeof(int32_t)) == hipSuccess;
+        if (ok) tmp_more.push_back(rows_in);
+        ok = ok && rocprim::radix_sort_pairs(nullptr, sort_bytes, tmp_mask[d], keys_out, rows_in, perm,
+                                             (size_t)n, 0u, (unsigned)k_vol, s) == hipSuccess;
+        ok = ok && hipMalloc(&sort_tmp, sort_bytes ? sort_bytes : 1) == hipSuccess;
+        if (ok) tmp_more.push_back(sort_tmp);
+        if (ok) {
+          iota_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(rows_in, (int)n);
+          ok = rocprim::radix_sort_pairs(sort_tmp, sort_bytes, tmp_mask[d], keys_out, rows_in, perm,
+                                         (size_t)n, 0u, (unsigned)k_vol, s) == hipSuccess;
+        }
+        if (!ok) {
+          (void)hipFree(sorted);
+          free_tmp();
+          set_error("fgms_plan_create: row sort failed");
+          return fail(FGMS_E_HIP);
+        }
         permute_table_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(tab, perm, (int)n, k_vol, sorted);
         tmp_tab[d] = tab;      // the unsorted table, freed after the sync
         tab = sorted;

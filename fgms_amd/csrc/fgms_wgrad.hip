@@ -223,7 +223,7 @@ template <> struct WTW<__half> { static constexpr int stage_pairs = 32; };
 template <> struct WTW<float> { static constexpr int stage_pairs = 16; };
 
 template <typename T, int BI, int BJ>
-__global__ __launch_bounds__(kThreads) void wgrad_wave_kernel(
+__global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
     const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk) {
