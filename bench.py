@@ -179,6 +179,27 @@ def main():
     recs = capi.profile_records()
     capi.profile_reset()
 
+    # gather-only pass over the rows the planned kernels read: the memory-side floor
+    gather_floor = None
+    if plan is not None and L["k_vol"] <= 64 and (L["c_in"] * D["in_feats"].element_size()) % 16 == 0 \
+            and (L["c_out"] * D["in_feats"].element_size()) % 16 == 0:
+        capi.profile_enable(True)
+        for _ in range(20):
+            if "fwd" in passes:
+                capi.probe_gather(D["in_feats"], plan, for_dgrad=False)
+            if "dgrad" in passes:
+                capi.probe_gather(D["out_grad"], plan, for_dgrad=True)
+        torch.cuda.synchronize()
+        capi.profile_enable(False)
+        pr = {}
+        for name, ms in capi.profile_records():
+            pr.setdefault(name, []).append(ms)
+        capi.profile_reset()
+        gather_floor = {k.replace("gather_probe_kernel", "").strip("()") + "_ms": sum(v[2:]) / len(v[2:])
+                        for k, v in pr.items()}
+        gather_floor["what"] = ("fgms_probe_gather: the same neighbour-table gathers as the planned kernel, "
+                                "nothing else (no weights, MFMA, LDS or result rows), all wave slots in use")
+
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = len(passes) * flops_pass / (ms_per_step * 1e-3) / 1e12
 
@@ -201,9 +222,13 @@ def main():
                         "avg_kernel_ms": kernels[dom]["avg_ms"]}
         else:
             ach = flops_pass / avg_s / 1e12
+            which = "dgrad" if "dgrad" in dom else ("wgrad" if "wgrad" in dom else "fwd")
             roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_TFLOPS[arith],
                         "unit": "TFLOP/s", "frac": ach / PEAK_TFLOPS[arith], "traffic": measured_traffic(args.workload, dom),
-                        "avg_kernel_ms": kernels[dom]["avg_ms"]}
+                        "avg_kernel_ms": kernels[dom]["avg_ms"],
+                        # the same launch priced as pair-list dataflow bytes against HBM
+                        "dataflow_bytes": dataflow_bytes(L, which),
+                        "dataflow_GBs": dataflow_bytes(L, which) / avg_s / 1e9}
 
     line = {
         "metric": "effective TFLOP/s (2*sum|map_k|*Cin*Cout/t), %s, %s"
@@ -216,6 +241,7 @@ def main():
                    "plan": plan is not None, "policy": args.policy},
         "kernels": kernels,
         "roofline": roofline,
+        "gather_floor": gather_floor,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload),
     }
     print(json.dumps(line))

@@ -19,7 +19,8 @@ LIB_DIR = os.path.join(ROOT, "fgms_amd", "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfgms_hip.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
-HIP_SOURCES = ["fgms_api.hip", "fgms_generic.hip", "fgms_plan.hip", "fgms_mfma.hip", "fgms_small.hip", "fgms_wgrad.hip"]
+HIP_SOURCES = ["fgms_api.hip", "fgms_generic.hip", "fgms_plan.hip", "fgms_mfma.hip", "fgms_small.hip", "fgms_wgrad.hip",
+               "fgms_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXX = os.environ.get("CXX", "g++")

@@ -17,7 +17,7 @@ SYMBOLS = [
     "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
-    "fgms_profile_reset",
+    "fgms_profile_reset", "fgms_probe_gather",
 ]
 
 _lib = None
@@ -50,6 +50,8 @@ def lib():
                            i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_dgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_wgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_probe_gather.argtypes = [vp, i32, i32, i32, vp, vp]
+    L.fgms_probe_gather.restype = i32
     L.fgms_set_kernel_policy.argtypes = [i32]
     L.fgms_set_kernel_policy.restype = None
     L.fgms_profile_enable.argtypes = [i32]
@@ -213,6 +215,12 @@ def dgrad(out_grad, kernel, in_grad, kpos, in_map, out_map, plan=None):
         _p(out_grad), _p(kernel), _p(in_grad), _p(kpos), _p(in_map), _p(out_map),
         in_grad.shape[0], out_grad.shape[0], kernel.shape[1], kernel.shape[2], kernel.shape[0],
         in_map.numel(), _dtype(out_grad), _ph(plan), _stream()))
+
+
+def probe_gather(feats, plan, for_dgrad=False):
+    """Gather-only pass over the rows the planned kernel reads (diagnostic)."""
+    _check(lib().fgms_probe_gather(_p(feats), feats.shape[1], _dtype(feats), int(for_dgrad),
+                                   _ph(plan), _stream()))
 
 
 def wgrad(in_feats, out_grad, kernel_grad, kpos, in_map, out_map, plan=None):

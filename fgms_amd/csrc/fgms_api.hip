@@ -293,7 +293,6 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
                const int32_t *kpos, const int32_t *in_map, const int32_t *out_map, int64_t n_in,
                int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype,
                fgms_plan_t *plan, void *stream) {
-  (void)plan;
   int rc = check_common(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
                         c_in, c_out, k_vol, n_pairs, dtype);
   if (rc) return rc;
@@ -302,6 +301,7 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
   a.imap = in_map; a.omap = out_map; a.n_in = n_in; a.n_out = n_out; a.c_in = c_in;
   a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
+  a.plan = (const Plan *)plan;
   return run_wgrad(a);
 }
 
@@ -316,6 +316,19 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
   if (rc) return rc;
   return fgms_wgrad(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
                     c_in, c_out, k_vol, n_pairs, dtype, plan, stream);
+}
+
+int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad, fgms_plan_t *plan,
+                      void *stream) {
+  const Plan *p = (const Plan *)plan;
+  if (!p || !feats || c_src <= 0 || (dtype != FGMS_F16 && dtype != FGMS_F32)) {
+    set_error("fgms_probe_gather: bad argument");
+    return FGMS_E_INVALID;
+  }
+  void *sink = nullptr;
+  int rc = workspace_get((hipStream_t)stream, 3, 256, &sink);
+  if (rc) return rc;
+  return launch_gather_probe(p, feats, c_src, dtype, for_dgrad != 0, sink, (hipStream_t)stream);
 }
 
 }  // extern "C"

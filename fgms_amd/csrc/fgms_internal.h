@@ -59,6 +59,7 @@ struct WgradArgs {
   int64_t n_pairs;
   int dtype;
   hipStream_t stream;
+  const struct Plan *plan;   // optional
 };
 
 // Plan: neighbour tables built from the pair lists.
@@ -78,13 +79,20 @@ struct Plan {
   // offset k (only built when k_vol <= 64; the output-stationary kernels need it)
   unsigned long long *mask_out;  // [ceil(n_out / 64)]
   unsigned long long *mask_in;   // [ceil(n_in / 64)]
+  // Row bands for the weight gradient: the output rows are cut into band_count
+  // equal bands and band_start[k * (band_count + 1) + c] is the first pair of
+  // offset k whose output row lies in band c or later (relative to kpos[k]).
+  // Only valid when every offset's pairs are ordered by output row (bands_ok).
+  int band_count;
+  int32_t *band_start;   // [k_vol, band_count + 1]
+  bool bands_ok;
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
 
 // Fp32 scratch that outlives a call (per device and stream, grown on demand).
 // slot 0: packed weights, slot 1: fp32 weight-gradient accumulator of the MFMA kernels (kept
-// all-zero between calls), slot 2: the generic kernel's accumulator.
+// all-zero between calls), slot 2: the generic kernel's accumulator, slot 3: the gather probe's sink.
 // *fresh (optional) is set when the buffer was (re)allocated by this call.
 int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *fresh = nullptr);
 size_t workspace_bytes(hipStream_t stream, int slot);
@@ -109,5 +117,7 @@ bool small_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_small_gms(const GmsArgs &a, const Plan *p);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_planned_gms(const GmsArgs &a, const Plan *p);
+int launch_gather_probe(const Plan *p, const void *src, int c_src, int dtype, bool for_dgrad,
+                        void *sink, hipStream_t stream);
 
 }  // namespace fgms

@@ -25,15 +25,16 @@ __global__ void fill_i32_kernel(int32_t *__restrict__ p, size_t n, int32_t v) {
 }
 
 // flags[0]: an index is out of range; flags[1]: two pairs of one offset share
-// an output row; flags[2]: two pairs of one offset share an input row.
+// an output row; flags[2]: two pairs of one offset share an input row;
+// flags[3]: inside some offset the pairs are not ordered by output row.
 __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
                                     const int32_t *__restrict__ imap,
-                                    const int32_t *__restrict__ omap, int k_vol, int n_in,
-                                    int n_out, int32_t *__restrict__ nbr_out,
+                                    const int32_t *__restrict__ omap, int k_vol, int n_pairs,
+                                    int n_in, int n_out, int32_t *__restrict__ nbr_out,
                                     int32_t *__restrict__ nbr_in, int *__restrict__ flags) {
   const int total = kpos[k_vol];
   int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= total) return;
+  if (j >= total || j >= n_pairs) return;
   // offset of pair j: the last k with kpos[k] <= j
   int lo = 0, hi = k_vol;
   while (hi - lo > 1) {
@@ -46,6 +47,7 @@ __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
     flags[0] = 1;
     return;
   }
+  if (j > kpos[k] && omap[j - 1] > o) flags[3] = 1;
   if (atomicCAS(&nbr_out[(size_t)k * n_out + o], -1, i) != -1) flags[1] = 1;
   if (atomicCAS(&nbr_in[(size_t)k * n_in + i], -1, o) != -1) flags[2] = 1;
 }
@@ -85,6 +87,27 @@ __global__ void row_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, in
 // The 64 rows a wave works on then use nearly the same offsets and whole
 // (block, offset) steps can be skipped: on a surface-like cloud of 200 k voxels
 // the number of such steps drops from 68.6 k to 36.7 k (33 k would be perfect).
+// band_start[k][c] = number of pairs of offset k whose output row is below
+// c * band_rows (a lower bound over the offset's pairs, which are ordered by
+// output row when the result is used); c = band_count gives the offset's size.
+__global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32_t *__restrict__ omap,
+                                   int n_pairs, int band_count, int band_rows,
+                                   int32_t *__restrict__ band_start) {
+  const int k = blockIdx.x;
+  const int first = min(max(kpos[k], 0), n_pairs);
+  const int count = min(max(kpos[k + 1], first), n_pairs) - first;   // never reads past the map
+  for (int c = threadIdx.x; c <= band_count; c += blockDim.x) {
+    int lo = 0, hi = count;              // first pair with omap >= c * band_rows
+    if (c == band_count) lo = count;
+    const long long target = (long long)c * band_rows;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (omap[first + mid] < target) lo = mid + 1; else hi = mid;
+    }
+    band_start[k * (band_count + 1) + c] = lo;
+  }
+}
+
 __global__ void iota_kernel(int32_t *__restrict__ p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = i;
@@ -134,6 +157,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->k_vol = k_vol; p->n_in = n_in; p->n_out = n_out; p->n_pairs = n_pairs;
   p->nbr_out = p->nbr_in = nullptr; p->mask_out = p->mask_in = nullptr;
   p->perm_out = p->perm_in = nullptr;
+  p->band_count = 0; p->band_start = nullptr; p->bands_ok = false;
   p->fwd_ok = p->dgrad_ok = false;
   int *flags = nullptr;
   int rc = FGMS_OK;
@@ -143,12 +167,27 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
     return code;
   };
   if (hipGetDevice(&p->device) != hipSuccess) return fail(FGMS_E_HIP);
+  // weight-gradient row bands: about 2048 output rows each but enough bands to
+  // fill the chip (bands x offsets >= ~1536 workgroups) and no more than leaves a
+  // workgroup ~400 pairs on average; a multiple of 8 (one per XCD), 8..kMaxBands
+  {
+    int64_t want = n_out / 2048;
+    const int64_t fill = (1536 + k_vol - 1) / k_vol;
+    if (want < fill) want = fill;
+    const int64_t by_work = n_pairs / ((int64_t)k_vol * 384);
+    if (want > by_work) want = by_work;
+    want = (want + 7) / 8 * 8;
+    constexpr int kMaxBands = 64;
+    p->band_count = (int)(want < 8 ? 8 : (want > kMaxBands ? kMaxBands : want));
+  }
+  const int band_rows = (int)((n_out + p->band_count - 1) / p->band_count);
   const size_t so = (size_t)n_out * k_vol, si = (size_t)n_in * k_vol;
   const size_t bo = (size_t)(n_out + 63) / 64, bi = (size_t)(n_in + 63) / 64;
   if (hipMalloc((void **)&p->nbr_out, (so ? so : 1) * sizeof(int32_t)) != hipSuccess ||
       hipMalloc((void **)&p->nbr_in, (si ? si : 1) * sizeof(int32_t)) != hipSuccess ||
       hipMalloc((void **)&p->mask_out, (bo ? bo : 1) * sizeof(unsigned long long)) != hipSuccess ||
       hipMalloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long)) != hipSuccess ||
+      hipMalloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t)) != hipSuccess ||
       hipMalloc((void **)&flags, 4 * sizeof(int)) != hipSuccess) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
@@ -158,12 +197,14 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   if ((rc = fill_i32(flags, 4, 0, s))) return fail(rc);
   if (n_pairs > 0) {
     build_tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
-        kpos, in_map, out_map, k_vol, (int)n_in, (int)n_out, p->nbr_out, p->nbr_in, flags);
+        kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, p->nbr_out, p->nbr_in, flags);
     if (hipGetLastError() != hipSuccess) {
       set_error("fgms_plan_create: table build launch failed");
       return fail(FGMS_E_HIP);
     }
   }
+  band_bounds_kernel<<<(unsigned)k_vol, 128, 0, s>>>(kpos, out_map, (int)n_pairs, p->band_count,
+                                                     band_rows > 0 ? band_rows : 1, p->band_start);
   // Reorder the rows (stable sort by offset mask), then derive the block masks
   // from the tables in their final order.  Temporaries are freed after the
   // stream synchronisation below.
@@ -251,6 +292,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   }
   p->fwd_ok = !h[1];
   p->dgrad_ok = !h[2];
+  p->bands_ok = !h[3];
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
 }
@@ -264,6 +306,7 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->mask_in) (void)hipFree(p->mask_in);
   if (p->perm_out) (void)hipFree(p->perm_out);
   if (p->perm_in) (void)hipFree(p->perm_in);
+  if (p->band_start) (void)hipFree(p->band_start);
   delete p;
 }
 

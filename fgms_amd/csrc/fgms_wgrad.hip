@@ -226,7 +226,8 @@ template <typename T, int BI, int BJ>
 __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk) {
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk,
+    const int32_t *__restrict__ band_start) {
   using W = WT<T>;
   constexpr int E = W::E, SP = WTW<T>::stage_pairs, KP = W::step_pairs;
   constexpr int CI = BI * 32, CO = BJ * 32;
@@ -235,20 +236,29 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
   constexpr int NX = SP * NCI / 64, NG = SP * NCO / 64;   // chunks per lane and stage
   static_assert(NX >= 1 && NG >= 1, "stage too small");
   extern __shared__ int4v lds[];
-  // Workgroup -> (slice c of the pair list, offset k).  Every offset is cut into
-  // the same number of slices, so slice c of each offset covers about the same
-  // band of rows (pair lists are ordered by row inside an offset).  Workgroups
-  // go to the 8 XCDs round-robin; numbering them so that one XCD gets all the
-  // offsets of a slice lets the rows one offset pulled into that XCD's L2 serve
-  // the other offsets of the slice.
+  // Workgroup -> (slice sl of the pair list, offset k).  Workgroups go to the 8
+  // XCDs round-robin; numbering them so that one XCD gets all the offsets of a
+  // slice lets the rows one offset pulled into that XCD's L2 serve the other
+  // offsets of the slice, provided slice sl of every offset covers the same band
+  // of rows.  With a plan whose pair lists are ordered by output row the slices
+  // are exactly such bands (band_start, found by bisection when the plan was
+  // built); without one every offset is cut into equal pair counts, which only
+  // approximates it.
   const int slices = chunk;               // (slices per offset, a multiple of 8)
   const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
   const int sl = (idx / k_vol) * 8 + xcd, k = idx % k_vol;
   if (sl >= slices) return;
   const int k_first = kpos[k], k_count = kpos[k + 1] - k_first;
-  const int per = (k_count + slices - 1) / slices;
-  const int first = k_first + sl * per;
-  const int count = min(per, k_count - sl * per);
+  int first, count;
+  if (band_start) {
+    const int b0 = band_start[k * (slices + 1) + sl], b1 = band_start[k * (slices + 1) + sl + 1];
+    first = k_first + b0;
+    count = b1 - b0;
+  } else {
+    const int per = (k_count + slices - 1) / slices;
+    first = k_first + sl * per;
+    count = min(per, k_count - sl * per);
+  }
   if (count <= 0) return;
   const int tiles_co = c_out / CO;
   const int ci0 = (blockIdx.y / tiles_co) * CI;
@@ -462,13 +472,22 @@ int launch_wave(const WgradArgs &a, float *acc32) {
   using W = WT<T>;
   constexpr int SP = WTW<T>::stage_pairs;
   const int ty = (a.c_in / (32 * BI)) * (a.c_out / (32 * BJ));
-  // slices per offset: enough workgroups to fill the chip a few times, at least
-  // ~16 stages of pairs per slice on average, a multiple of 8 (one per XCD)
-  int64_t slices = (int64_t)num_cus() * 6 / ((int64_t)a.k_vol * ty);
-  const int64_t by_work = a.n_pairs / ((int64_t)a.k_vol * 16 * SP);
-  if (slices > by_work) slices = by_work;
-  slices = (slices + 7) / 8 * 8;
-  if (slices < 8) slices = 8;
+  // slices per offset: the plan's row bands when it has them; else enough
+  // workgroups to fill the chip a few times, at least ~16 stages of pairs per
+  // slice on average, a multiple of 8 (one per XCD)
+  const int32_t *band_start = nullptr;
+  int64_t slices;
+  if (a.plan && a.plan->bands_ok && a.plan->band_start && a.plan->k_vol == a.k_vol &&
+      a.plan->n_pairs == a.n_pairs && a.plan->n_out == a.n_out) {
+    slices = a.plan->band_count;
+    band_start = a.plan->band_start;
+  } else {
+    slices = (int64_t)num_cus() * 6 / ((int64_t)a.k_vol * ty);
+    const int64_t by_work = a.n_pairs / ((int64_t)a.k_vol * 16 * SP);
+    if (slices > by_work) slices = by_work;
+    slices = (slices + 7) / 8 * 8;
+    if (slices < 8) slices = 8;
+  }
   const int64_t chunk = slices;
   const int64_t tiles = slices * a.k_vol;
   size_t lds = 4 * (size_t)SP * ((BI * 32 + W::pad) + (BJ * 32 + W::pad)) * sizeof(T);
@@ -481,7 +500,7 @@ int launch_wave(const WgradArgs &a, float *acc32) {
     ProfileScope prof("wgrad_wave_kernel", a.stream);
     kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
-        a.c_out, (int)chunk);
+        a.c_out, (int)chunk, band_start);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;

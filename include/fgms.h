@@ -134,6 +134,19 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
 void fgms_set_kernel_policy(int policy);
 
 /*
+ * Diagnostic, no counterpart in the reference: reads exactly the feature rows
+ * the output-stationary forward (for_dgrad = 0: feats = in_feats, c_src = c_in)
+ * or input-gradient kernel (for_dgrad != 0: feats = out_feats_grad,
+ * c_src = c_out) gathers for this plan, and nothing else: no weights, no
+ * matrix cores, no result.  Timed through fgms_profile_* it gives the time the
+ * memory system alone needs for the gathers of one pass, the floor that the
+ * real kernel's duration is compared with.  Rows must be 16 * 2^j bytes
+ * (j = 0..6); k_vol <= 64.
+ */
+int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad,
+                      fgms_plan_t *plan, void *stream);
+
+/*
  * Per-kernel timing with HIP events on the stream the kernels are launched on
  * (no counterpart in the reference, which times whole calls from python,
  * spconv-test.py:95-122).  While enabled, every main kernel launch (not the

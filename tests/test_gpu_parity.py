@@ -213,3 +213,24 @@ def test_config2_scaled_fp32_and_tf32(capi, oracle):
     L = clouds.config_case(2, scale=0.08)
     check_all(capi, oracle, L, policy=0, use_plan=True, arch80=False)
     check_all(capi, oracle, L, policy=0, use_plan=True, arch80=True)
+
+
+def test_gather_probe_runs_and_is_timed(capi):
+    """The diagnostic gather-only pass: launches over a plan for both directions,
+    leaves the tensors untouched and shows up in the per-kernel timing records."""
+    L = layer(31, 64, 32, np.float16)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    before_in, before_g = D["in_feats"].clone(), D["out_grad"].clone()
+    capi.profile_reset()
+    capi.profile_enable(True)
+    capi.probe_gather(D["in_feats"], plan, for_dgrad=False)
+    capi.probe_gather(D["out_grad"], plan, for_dgrad=True)
+    torch.cuda.synchronize()
+    capi.profile_enable(False)
+    names = [n for n, _ in capi.profile_records()]
+    capi.profile_reset()
+    assert names == ["gather_probe_kernel(fwd)", "gather_probe_kernel(dgrad)"]
+    assert torch.equal(before_in, D["in_feats"]) and torch.equal(before_g, D["out_grad"])
+    with pytest.raises(ValueError):
+        capi.probe_gather(D["in_feats"][:, :3].contiguous(), plan)     # 6-byte rows
