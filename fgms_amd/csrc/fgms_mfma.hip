@@ -360,7 +360,7 @@ __device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (
 }
 
 template <typename T, int NT, int S>
-__global__ __launch_bounds__(kThreads, 3) void gms_rows_kernel(
+__global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, int n_dst, int k_vol, int c_src, int c_dst) {
@@ -482,6 +482,7 @@ __global__ __launch_bounds__(kThreads, 3) void gms_rows_kernel(
 // ---------------------------------------------------------------------------
 struct Shape {
   int c_src, c_dst, S, NT, E;
+  int NTR;                // 32-column tiles per wave in the output-stationary kernel
   size_t lds_bytes;       // pair-stationary kernel
   size_t lds_rows_bytes;  // output-stationary kernel
   bool ok;
@@ -502,7 +503,13 @@ Shape shape_of(const GmsArgs &a) {
   const size_t tiles = (size_t)kWaves * kWaveRows * 2 * s.S * 16  // staging tiles
                        + (size_t)kWaves * 2 * kWaveRows * sizeof(int);
   s.lds_bytes = (size_t)s.c_src * s.NT * 32 * esz + tiles;      // + weights of one offset
-  s.lds_rows_bytes = 2 * (size_t)s.S * s.NT * 64 * 16 + tiles;  // + two stages of weights
+  // wide fp16 layers: 128 columns per wave, so that a row is gathered once per 128
+  // (not 64) output channels.  Costs 128 accumulator registers (2 waves per SIMD)
+  // and halves the number of workgroups, so only when enough of them remain to
+  // fill the chip; fp32 has 8x the MFMA time per gathered byte and gains nothing.
+  const int64_t wide_wgs = (a.n_dst + kTileRows - 1) / kTileRows * (s.c_dst / 128);
+  s.NTR = (a.dtype == FGMS_F16 && s.c_dst % 128 == 0 && wide_wgs * 2 >= 3 * (int64_t)num_cus()) ? 4 : s.NT;
+  s.lds_rows_bytes = 2 * (size_t)s.S * s.NTR * 64 * 16 + tiles;  // + two stages of weights
   s.ok = s.lds_bytes <= 128 * 1024;
   return s;
 }
@@ -568,6 +575,19 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
+}
+
+template <typename T, typename F>
+int dispatch_shape(const Shape &s, F &&f);
+
+template <typename T, typename F>
+int dispatch_rows_shape(const Shape &s, F &&f) {
+  if (s.NTR == 4) {
+    if (s.S == 4) return f(std::integral_constant<int, 4>{}, std::integral_constant<int, 4>{});
+    if (s.S == 2) return f(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+    return f(std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{});
+  }
+  return dispatch_shape<T>(s, f);
 }
 
 template <typename T, typename F>
@@ -648,10 +668,10 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p) {
   const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
   const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
   if (a.dtype == FGMS_F16)
-    return dispatch_shape<__half>(s, [&](auto nt, auto sv) {
+    return dispatch_rows_shape<__half>(s, [&](auto nt, auto sv) {
       return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm);
     });
-  return dispatch_shape<float>(s, [&](auto nt, auto sv) {
+  return dispatch_rows_shape<float>(s, [&](auto nt, auto sv) {
     return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm);
   });
 }

@@ -67,11 +67,47 @@ __device__ __forceinline__ half8 tr_frag(const __half *tile, int ld, int p0, int
   return __builtin_bit_cast(half8, v);
 }
 
+// Workgroup -> (slice sl of the pair list, offset k) and the slice's pair range.
+// Workgroups go to the 8 XCDs round-robin; numbering them so that one XCD gets
+// all the offsets of a slice lets the rows one offset pulled into that XCD's L2
+// serve the other offsets of the slice, provided slice sl of every offset covers
+// the same band of rows.  With a plan whose pair lists are ordered by output row
+// a slice is `stride` consecutive row bands of the plan (band_start, found by
+// bisection when the plan was built); without one every offset is cut into equal
+// pair counts, which only approximates it.  slices is a multiple of 8.
+struct SliceMap {
+  const int32_t *band_start;   // [k_vol][bands + 1] or nullptr
+  int bands, stride;           // slice sl = bands [sl * stride, (sl + 1) * stride)
+  int slices;
+  int chunk;                   // > 0: plain tiles of `chunk` pairs in pair-list order instead
+};
+
+__device__ __forceinline__ bool locate_slice(const int32_t *__restrict__ kpos, const SliceMap &m,
+                                             int k_vol, int block, int &k, int &first, int &count) {
+  if (m.chunk > 0) return locate_tile(kpos, k_vol, m.chunk, block, k, first, count);
+  const int xcd = block % 8, idx = block / 8;
+  const int sl = (idx / k_vol) * 8 + xcd;
+  k = idx % k_vol;
+  if (sl >= m.slices) return false;
+  const int k_first = kpos[k], k_count = kpos[k + 1] - k_first;
+  if (m.band_start) {
+    const int32_t *row = m.band_start + (size_t)k * (m.bands + 1);
+    const int b0 = row[min(sl * m.stride, m.bands)], b1 = row[min((sl + 1) * m.stride, m.bands)];
+    first = k_first + b0;
+    count = b1 - b0;
+  } else {
+    const int per = (k_count + m.slices - 1) / m.slices;
+    first = k_first + sl * per;
+    count = min(per, k_count - sl * per);
+  }
+  return count > 0;
+}
+
 template <typename T, int BI, int BJ>
 __global__ __launch_bounds__(kThreads) void wgrad_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk) {
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap) {
   using W = WT<T>;
   using G = WaveGrid<BI, BJ>;
   constexpr int E = W::E, SP = W::stage_pairs, KP = W::step_pairs;
@@ -87,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
   gs[1] = xs[1] + SP * LDI;
 
   int k, first, count;
-  if (!locate_tile(kpos, k_vol, chunk, blockIdx.x, k, first, count)) return;
+  if (!locate_slice(kpos, smap, k_vol, blockIdx.x, k, first, count)) return;
   const int tiles_co = c_out / CO;
   const int ci0 = (blockIdx.y / tiles_co) * CI;
   const int co0 = (blockIdx.y % tiles_co) * CO;
@@ -226,8 +262,7 @@ template <typename T, int BI, int BJ>
 __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, int chunk,
-    const int32_t *__restrict__ band_start) {
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap) {
   using W = WT<T>;
   constexpr int E = W::E, SP = WTW<T>::stage_pairs, KP = W::step_pairs;
   constexpr int CI = BI * 32, CO = BJ * 32;
@@ -236,30 +271,8 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
   constexpr int NX = SP * NCI / 64, NG = SP * NCO / 64;   // chunks per lane and stage
   static_assert(NX >= 1 && NG >= 1, "stage too small");
   extern __shared__ int4v lds[];
-  // Workgroup -> (slice sl of the pair list, offset k).  Workgroups go to the 8
-  // XCDs round-robin; numbering them so that one XCD gets all the offsets of a
-  // slice lets the rows one offset pulled into that XCD's L2 serve the other
-  // offsets of the slice, provided slice sl of every offset covers the same band
-  // of rows.  With a plan whose pair lists are ordered by output row the slices
-  // are exactly such bands (band_start, found by bisection when the plan was
-  // built); without one every offset is cut into equal pair counts, which only
-  // approximates it.
-  const int slices = chunk;               // (slices per offset, a multiple of 8)
-  const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
-  const int sl = (idx / k_vol) * 8 + xcd, k = idx % k_vol;
-  if (sl >= slices) return;
-  const int k_first = kpos[k], k_count = kpos[k + 1] - k_first;
-  int first, count;
-  if (band_start) {
-    const int b0 = band_start[k * (slices + 1) + sl], b1 = band_start[k * (slices + 1) + sl + 1];
-    first = k_first + b0;
-    count = b1 - b0;
-  } else {
-    const int per = (k_count + slices - 1) / slices;
-    first = k_first + sl * per;
-    count = min(per, k_count - sl * per);
-  }
-  if (count <= 0) return;
+  int k, first, count;
+  if (!locate_slice(kpos, smap, k_vol, blockIdx.x, k, first, count)) return;
   const int tiles_co = c_out / CO;
   const int ci0 = (blockIdx.y / tiles_co) * CI;
   const int co0 = (blockIdx.y % tiles_co) * CO;
@@ -441,18 +454,50 @@ int num_cus() {
   return cus;
 }
 
+// Slices per offset: from the plan's row bands when it has them, `stride` bands to
+// a slice so that about `want_wgs` workgroups result; else equal pair counts,
+// enough to fill the chip a few times with at least ~16 stages of pairs per slice
+// on average.  A multiple of 8 (one per XCD).
+SliceMap choose_slices(const WgradArgs &a, int ty, int stage_pairs, int64_t want_wgs) {
+  SliceMap m{};
+  if (a.plan && a.plan->bands_ok && a.plan->band_start && a.plan->k_vol == a.k_vol &&
+      a.plan->n_pairs == a.n_pairs && a.plan->n_out == a.n_out) {
+    m.band_start = a.plan->band_start;
+    m.bands = a.plan->band_count;
+    m.stride = 1;
+    while (m.stride < 8 && (int64_t)(m.bands / (m.stride * 2)) * a.k_vol * ty >= want_wgs &&
+           (m.bands / (m.stride * 2)) % 8 == 0)
+      m.stride *= 2;
+    m.slices = (m.bands + m.stride - 1) / m.stride;
+    return m;
+  }
+  int64_t slices = want_wgs / ((int64_t)a.k_vol * ty);
+  const int64_t by_work = a.n_pairs / ((int64_t)a.k_vol * 16 * stage_pairs);
+  if (slices > by_work) slices = by_work;
+  slices = (slices + 7) / 8 * 8;
+  m.slices = (int)(slices < 8 ? 8 : slices);
+  return m;
+}
+
 template <typename T, int BI, int BJ>
 int launch(const WgradArgs &a, float *acc32) {
   using W = WT<T>;
   constexpr int SP = W::stage_pairs;
   const int ty = (a.c_in / (32 * BI)) * (a.c_out / (32 * BJ));
-  // enough workgroups to fill the chip a few times over, chunks a multiple of the stage size
-  int64_t want = (int64_t)num_cus() * 4 / ty;
-  if (want < 1) want = 1;
-  int64_t chunk = (a.n_pairs + want - 1) / want;
-  chunk = (chunk + SP - 1) / SP * SP;
-  if (chunk < 4 * SP) chunk = 4 * SP;
-  const int64_t tiles = (a.n_pairs + chunk - 1) / chunk + a.k_vol;
+  SliceMap smap{};
+  int64_t tiles;
+  if (BI * BJ == 16) {
+    // whole 128 x 128 tiles (64 KB to flush per workgroup, 2 workgroups per CU):
+    // equal tiles in pair-list order, about 4 per CU, measured faster than row bands
+    int64_t chunk = (a.n_pairs + (int64_t)num_cus() * 4 - 1) / ((int64_t)num_cus() * 4);
+    chunk = (chunk + SP - 1) / SP * SP;
+    if (chunk < 4 * SP) chunk = 4 * SP;
+    smap.chunk = (int)chunk;
+    tiles = (a.n_pairs + chunk - 1) / chunk + a.k_vol;
+  } else {
+    smap = choose_slices(a, ty, SP, (int64_t)num_cus() * 4);
+    tiles = (int64_t)smap.slices * a.k_vol;
+  }
   const size_t lds = 2 * (size_t)SP * ((BI * 32 + W::pad) + (BJ * 32 + W::pad)) * sizeof(T);
   auto kern = wgrad_kernel<T, BI, BJ>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -461,7 +506,7 @@ int launch(const WgradArgs &a, float *acc32) {
     ProfileScope prof("wgrad_kernel", a.stream);
     kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
-        a.c_out, (int)chunk);
+        a.c_out, smap);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -472,24 +517,8 @@ int launch_wave(const WgradArgs &a, float *acc32) {
   using W = WT<T>;
   constexpr int SP = WTW<T>::stage_pairs;
   const int ty = (a.c_in / (32 * BI)) * (a.c_out / (32 * BJ));
-  // slices per offset: the plan's row bands when it has them; else enough
-  // workgroups to fill the chip a few times, at least ~16 stages of pairs per
-  // slice on average, a multiple of 8 (one per XCD)
-  const int32_t *band_start = nullptr;
-  int64_t slices;
-  if (a.plan && a.plan->bands_ok && a.plan->band_start && a.plan->k_vol == a.k_vol &&
-      a.plan->n_pairs == a.n_pairs && a.plan->n_out == a.n_out) {
-    slices = a.plan->band_count;
-    band_start = a.plan->band_start;
-  } else {
-    slices = (int64_t)num_cus() * 6 / ((int64_t)a.k_vol * ty);
-    const int64_t by_work = a.n_pairs / ((int64_t)a.k_vol * 16 * SP);
-    if (slices > by_work) slices = by_work;
-    slices = (slices + 7) / 8 * 8;
-    if (slices < 8) slices = 8;
-  }
-  const int64_t chunk = slices;
-  const int64_t tiles = slices * a.k_vol;
+  const SliceMap smap = choose_slices(a, ty, SP, (int64_t)num_cus() * 6);
+  const int64_t tiles = (int64_t)smap.slices * a.k_vol;
   size_t lds = 4 * (size_t)SP * ((BI * 32 + W::pad) + (BJ * 32 + W::pad)) * sizeof(T);
   const size_t red = 2 * (size_t)BI * BJ * 16 * 64 * sizeof(float);
   if (lds < red) lds = red;
@@ -500,7 +529,7 @@ int launch_wave(const WgradArgs &a, float *acc32) {
     ProfileScope prof("wgrad_wave_kernel", a.stream);
     kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
-        a.c_out, (int)chunk, band_start);
+        a.c_out, smap);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
