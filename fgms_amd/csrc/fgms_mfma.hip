@@ -252,6 +252,78 @@ __device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__rest
   }
 }
 
+// The same update with the tile transposed through the wave's own LDS staging
+// region (free once the last MFMAs have read it): accumulators go to LDS as fp32,
+// R rows at a time, and come back row-major, so every lane adds 4 consecutive
+// columns of one row and a destination row is read and written as whole
+// 64..256-byte runs by neighbouring lanes instead of 4 bytes per lane.
+// stage: the wave's staging tile, 64 * 2*S * 16 bytes.
+template <typename T, int NT, int S>
+__device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__restrict__ dst,
+                                             const int *__restrict__ rows, float *__restrict__ stage,
+                                             int c_dst, int cd0, int lane) {
+  constexpr int COLS = NT * 32;
+  constexpr int R = (64 * 2 * S * 16) / (COLS * 4) >= 32 ? 32 : (64 * 2 * S * 16) / (COLS * 4);
+  if constexpr (R < 8) {
+    add_rows<T, NT>(acc, dst, rows, c_dst, cd0, lane);
+  } else {
+    constexpr int CH = COLS / 4;            // 16-byte chunks per staged row
+    constexpr int IT = R * CH / 64;         // chunks per lane and pass
+    const int h = lane / 32, col = lane % 32;
+#pragma unroll
+    for (int p = 0; p < 64 / R; ++p) {
+      const int mt = (p * R) / 32, g0 = ((p * R) % 32) / 8;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int g = 0; g < R / 8; ++g)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            stage[(g * 8 + h * 4 + j) * COLS + nt * 32 + col] = acc[mt][nt][(g0 + g) * 4 + j];
+      wave_lds_fence();
+      float4v part[IT];
+      int row[IT];
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {
+        const int e = it * 64 + lane;
+        part[it] = *reinterpret_cast<const float4v *>(stage + (e / CH) * COLS + (e % CH) * 4);
+        row[it] = rows[p * R + e / CH];
+      }
+      if constexpr (sizeof(T) == 4) {
+        float4v old[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+          old[it] = *reinterpret_cast<const float4v *>(
+              reinterpret_cast<const float *>(dst) + (size_t)max(row[it], 0) * c_dst + cd0 +
+              ((it * 64 + lane) % CH) * 4);
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+          if (row[it] >= 0)
+            *reinterpret_cast<float4v *>(reinterpret_cast<float *>(dst) + (size_t)row[it] * c_dst + cd0 +
+                                         ((it * 64 + lane) % CH) * 4) = old[it] + part[it];
+      } else {
+        typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+        half4 old[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+          old[it] = *reinterpret_cast<const half4 *>(
+              reinterpret_cast<const _Float16 *>(dst) + (size_t)max(row[it], 0) * c_dst + cd0 +
+              ((it * 64 + lane) % CH) * 4);
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+          half4 out;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) out[q] = (_Float16)((float)old[it][q] + part[it][q]);
+          if (row[it] >= 0)
+            *reinterpret_cast<half4 *>(reinterpret_cast<_Float16 *>(dst) + (size_t)row[it] * c_dst + cd0 +
+                                       ((it * 64 + lane) % CH) * 4) = out;
+        }
+      }
+      wave_lds_fence();
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Pair-stationary kernel.
 template <typename T, int NT, int S>
@@ -475,7 +547,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   }
   if (wave_mask) {
     wave_lds_fence();
-    add_rows<T, NT>(acc, dst, didx, c_dst, nt0 * 32, lane);
+    add_rows_lds<T, NT, S>(acc, dst, didx, reinterpret_cast<float *>(a_lds), c_dst, nt0 * 32, lane);
   }
 }
 
@@ -655,6 +727,8 @@ bool planned_gms_supported(const GmsArgs &a, const Plan *p) {
   } else {
     if (!p->fwd_ok || a.n_dst != p->n_out || a.n_src != p->n_in) return false;
   }
+  // result rows are updated with 8- and 16-byte accesses
+  if (reinterpret_cast<uintptr_t>(a.dst) % 16) return false;
   return shape_of(a).ok;
 }
 
