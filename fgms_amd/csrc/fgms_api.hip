@@ -15,6 +15,7 @@ namespace fgms {
 
 static thread_local char g_error[512] = "";
 static int g_policy = 0;
+int kernel_policy() { return g_policy; }
 
 void set_error(const char *fmt, ...) {
   va_list ap;

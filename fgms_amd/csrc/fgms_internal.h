@@ -110,6 +110,7 @@ int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
 int launch_generic_gms(const GmsArgs &a);
 int launch_generic_wgrad(const WgradArgs &a);
 bool mfma_gms_supported(const GmsArgs &a);
+int kernel_policy();   // fgms_set_kernel_policy's value
 int launch_mfma_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);

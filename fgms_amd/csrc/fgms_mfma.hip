@@ -580,7 +580,8 @@ Shape shape_of(const GmsArgs &a) {
   // and halves the number of workgroups, so only when enough of them remain to
   // fill the chip; fp32 has 8x the MFMA time per gathered byte and gains nothing.
   const int64_t wide_wgs = (a.n_dst + kTileRows - 1) / kTileRows * (s.c_dst / 128);
-  s.NTR = (a.dtype == FGMS_F16 && s.c_dst % 128 == 0 && wide_wgs * 2 >= 3 * (int64_t)num_cus()) ? 4 : s.NT;
+  const bool wide = kernel_policy() == 3 || (a.dtype == FGMS_F16 && wide_wgs * 2 >= 3 * (int64_t)num_cus());
+  s.NTR = (s.c_dst % 128 == 0 && wide) ? 4 : s.NT;
   s.lds_rows_bytes = 2 * (size_t)s.S * s.NTR * 64 * 16 + tiles;  // + two stages of weights
   s.ok = s.lds_bytes <= 128 * 1024;
   return s;

@@ -130,7 +130,10 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
 
 /* Selects kernels by hand for tests and profiling: 0 = automatic dispatch,
  * 1 = force the generic (non-MFMA) kernels, 2 = force the pair-stationary MFMA
- * kernels even when a usable plan is passed.  Process-wide. */
+ * kernels even when a usable plan is passed, 3 = automatic dispatch but the
+ * output-stationary kernel uses its 128-column wave tiles whenever the layer
+ * has a multiple of 128 output channels (normally only large fp16 layers).
+ * Process-wide. */
 void fgms_set_kernel_policy(int policy);
 
 /*

@@ -83,6 +83,14 @@ def test_submanifold_pair_stationary_mfma(capi, oracle, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("shape", [(128, 128), (64, 128), (256, 256), (16, 128)], ids=lambda s: "%dx%d" % s)
+def test_submanifold_wide_wave_tiles(capi, oracle, shape, dtype):
+    """The 128-column wave tiles of the output-stationary kernel, which the automatic
+    dispatch reserves for large fp16 layers, forced on at test size."""
+    check_all(capi, oracle, layer(14, shape[0], shape[1], dtype), policy=3, use_plan=True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
 @pytest.mark.parametrize("kind,shape", [("down", (64, 128)), ("up", (128, 64)), ("down", (16, 32)), ("up", (5, 3))])
 def test_strided_and_transposed(capi, oracle, kind, shape, dtype):
     L = layer(14, shape[0], shape[1], dtype, kind)
@@ -234,3 +242,38 @@ def test_gather_probe_runs_and_is_timed(capi):
     assert torch.equal(before_in, D["in_feats"]) and torch.equal(before_g, D["out_grad"])
     with pytest.raises(ValueError):
         capi.probe_gather(D["in_feats"][:, :3].contiguous(), plan)     # 6-byte rows
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+def test_pairs_in_any_order_inside_an_offset(capi, oracle, dtype):
+    """The reference fixes no order of the pairs inside an offset.  Shuffled lists
+    make the plan drop its output-row bands (the weight gradient then slices by
+    pair count); every result must stay the same."""
+    L = layer(15, 64, 64, dtype)
+    rng = np.random.default_rng(15)
+    kpos = np.concatenate([[0], np.cumsum(L["knnz"])])
+    for k in range(L["k_vol"]):
+        p = kpos[k] + rng.permutation(kpos[k + 1] - kpos[k])
+        L["imap"][kpos[k]:kpos[k + 1]] = L["imap"][p]
+        L["omap"][kpos[k]:kpos[k + 1]] = L["omap"][p]
+    check_all(capi, oracle, L, policy=0, use_plan=True)
+    check_all(capi, oracle, L, policy=0, use_plan=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["fp32", "fp16"])
+def test_result_rows_not_16_byte_aligned(capi, oracle, dtype):
+    """A result tensor that starts 4 bytes (fp16) / 8 bytes (fp32) past a 16-byte
+    boundary cannot take the planned kernel's vector updates: the call must fall
+    back to the pair-stationary kernels and still be right."""
+    L = layer(16, 64, 64, np.float16 if dtype == torch.float16 else np.float32)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    buf = torch.zeros(D["n_out"] * 64 + 8, dtype=dtype, device="cuda")
+    out = buf[2:2 + D["n_out"] * 64].view(D["n_out"], 64)
+    assert out.data_ptr() % 16 != 0 and out.is_contiguous()
+    capi.fusion_fwd(D["in_feats"], D["kernel"], 0, out, D["kpos"], None, D["imap"], D["omap"],
+                    False, False, plan=plan)
+    torch.cuda.synchronize()
+    ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
+    G.assert_close(out.cpu().numpy(), ref, G.mode_of(dtype), "fwd into an unaligned result")
+    assert not buf[:2].any() and not buf[2 + D["n_out"] * 64:].any()
