@@ -1,0 +1,95 @@
+"""GPU checks at the full BASELINE sizes, where the CPU oracle is too slow to be the
+checker for every case: size-independent properties of the three products.
+
+With T(x, W, g) = sum_j  g[omap[j]] . (x[imap[j]] @ W[k(j)])  (a trilinear form):
+    <g, fwd(x, W)>  =  <dgrad(g, W), x>  =  <wgrad(x, g), W>  =  T(x, W, g)
+so the three kernels must agree on one number; forward is linear in x; the planned
+(output-stationary) and the pair-stationary kernels must agree with each other; and on
+the one configuration the C oracle finishes in a second it is compared directly."""
+import numpy as np
+import pytest
+import torch
+
+from fgms_amd import clouds
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from fgms_amd import capi as c
+    c.lib()
+    assert torch.cuda.is_available()
+    yield c
+    c.set_kernel_policy(0)
+
+
+def run_all(capi, D, plan):
+    dt = D["in_feats"].dtype
+    out = torch.zeros(D["n_out"], D["c_out"], dtype=dt, device="cuda")
+    gi = torch.zeros(D["n_in"], D["c_in"], dtype=dt, device="cuda")
+    gw = torch.zeros_like(D["kernel"])
+    capi.fusion_fwd(D["in_feats"], D["kernel"], 0, out, D["kpos"], None, D["imap"], D["omap"],
+                    False, False, plan=plan)
+    capi.dgrad(D["out_grad"], D["kernel"], gi, D["kpos"], D["imap"], D["omap"], plan=plan)
+    capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
+    torch.cuda.synchronize()
+    return out, gi, gw
+
+
+def dot(a, b):
+    return float((a.double() * b.double()).sum())
+
+
+CASES = [(2, "fp16", 2e-3), (2, None, 2e-5), (3, None, 2e-3), (4, None, 2e-3), (4, "up", 2e-3), (5, "wide", 2e-3)]
+
+
+@pytest.mark.parametrize("cfg,variant,tol", CASES, ids=lambda v: str(v))
+def test_trilinear_form_agrees_full_size(capi, cfg, variant, tol):
+    L = clouds.config_case(cfg, variant, scale=1.0)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    out, gi, gw = run_all(capi, D, plan)
+    t_f, t_d, t_w = dot(D["out_grad"], out), dot(gi, D["in_feats"]), dot(gw, D["kernel"])
+    # scale of the form: sqrt(#terms) * typical term, from the forward result itself
+    scale = float(out.double().norm() * D["out_grad"].double().norm())
+    assert abs(t_f - t_d) <= tol * scale, (t_f, t_d, scale)
+    assert abs(t_f - t_w) <= tol * scale, (t_f, t_w, scale)
+    assert torch.isfinite(out).all() and torch.isfinite(gi).all() and torch.isfinite(gw).all()
+
+    # linearity: fwd(2 x) = 2 fwd(x) bit for bit, scaling by two being exact, except where
+    # the fp16 result is subnormal (there the doubled sum keeps one more bit)
+    D2 = dict(D)
+    D2["in_feats"] = D["in_feats"] * 2
+    out2 = torch.zeros_like(out)
+    capi.fusion_fwd(D2["in_feats"], D["kernel"], 0, out2, D["kpos"], None, D["imap"], D["omap"],
+                    False, False, plan=plan)
+    torch.cuda.synchronize()
+    if out.dtype == torch.float16:
+        assert float((out2.float() - 2 * out.float()).abs().max()) <= 2.0 ** -23
+        normal = out.abs() > 2.0 ** -14      # 2^-14 itself can be a subnormal-range sum rounded up
+        assert torch.equal(out2[normal], (out * 2)[normal])
+    else:
+        assert torch.equal(out2, out * 2)
+
+    # the pair-stationary (atomic) kernels, no plan: same results within the mode's tolerance
+    mode = G.mode_of(D["in_feats"].dtype)
+    out_p, gi_p, gw_p = run_all(capi, D, None)
+    G.assert_close(out_p.cpu().numpy(), out.cpu().numpy(), mode, "fwd planned vs pair-stationary")
+    G.assert_close(gi_p.cpu().numpy(), gi.cpu().numpy(), mode, "dgrad planned vs pair-stationary")
+    G.assert_close(gw_p.cpu().numpy(), gw.cpu().numpy(), mode, "wgrad bands vs equal slices")
+    plan.close()
+
+
+def test_config1_full_size_against_oracle(capi, oracle):
+    """20 k voxels, 32 -> 32 fp32: small enough for the C oracle at full size."""
+    L = clouds.config_case(1, None, scale=1.0)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    out, gi, gw = run_all(capi, D, plan)
+    a = (L["knnz"], L["imap"], L["omap"])
+    G.assert_close(out.cpu().numpy(), oracle.c_fwd(L["in_feats"], L["kernel"], *a, L["n_out"]), "fp32", "fwd")
+    G.assert_close(gi.cpu().numpy(), oracle.c_dgrad(L["out_grad"], L["kernel"], *a, L["n_in"]), "fp32", "dgrad")
+    G.assert_close(gw.cpu().numpy(), oracle.c_wgrad(L["in_feats"], L["out_grad"], *a, L["k_vol"]), "fp32", "wgrad")
+    plan.close()
