@@ -123,6 +123,8 @@ def main():
     ap.add_argument("--no-plan", action="store_true", help="do not pass a kernel-map plan")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--scale", type=float, default=1.0, help="voxel-count scale (1.0 = the named size)")
+    ap.add_argument("--map-build", action="store_true",
+                    help="also time the device kernel-map builder and the plan build on the headline cloud")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run plain 256 MiB device copies (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -200,6 +202,41 @@ def main():
         gather_floor["what"] = ("fgms_probe_gather: the same neighbour-table gathers as the planned kernel, "
                                 "nothing else (no weights, MFMA, LDS or result rows), all wave slots in use")
 
+    # the steps before the path: pair lists from coordinates, plan from pair lists
+    map_build = None
+    if args.map_build:
+        import numpy as np
+        from fgms_amd import clouds
+        vox = torch.from_numpy(np.ascontiguousarray(clouds.indoor_cloud())).cuda()
+        offs = clouds.offsets_cube(3)
+        for _ in range(3):
+            capi.build_kernel_map(vox, vox, offs)
+        capi.profile_enable(True)
+        torch.cuda.synchronize()
+        tb = time.perf_counter()
+        for _ in range(10):
+            im_, om_, kn_, kp_ = capi.build_kernel_map(vox, vox, offs)
+        torch.cuda.synchronize()
+        t_map = (time.perf_counter() - tb) / 10
+        capi.profile_enable(False)
+        pr = {}
+        for name, ms in capi.profile_records():
+            pr.setdefault(name, []).append(ms)
+        capi.profile_reset()
+        tb = time.perf_counter()
+        for _ in range(10):
+            capi.Plan(kp_, im_, om_, vox.shape[0], vox.shape[0]).close()
+        torch.cuda.synchronize()
+        t_plan = (time.perf_counter() - tb) / 10
+        nbytes = 2 * vox.numel() * 4 + 2 * im_.numel() * 4     # coordinates read, pair lists written
+        k_ms = {k: sum(v) / len(v) for k, v in pr.items()}
+        map_build = {"voxels": int(vox.shape[0]), "pairs": int(im_.numel()), "k_vol": 27,
+                     "build_kernel_map_ms": t_map * 1e3, "kernels_ms": k_ms,
+                     "algorithmic_GBs": nbytes / (sum(k_ms.values()) * 1e-3) / 1e9,
+                     "plan_create_ms": t_plan * 1e3,
+                     "note": "wall clock per call incl. temporary allocations and the one synchronisation; "
+                             "algorithmic bytes = coordinates read + pair lists written"}
+
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = len(passes) * flops_pass / (ms_per_step * 1e-3) / 1e12
 
@@ -242,6 +279,7 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
         "gather_floor": gather_floor,
+        "map_build": map_build,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload),
     }
     print(json.dumps(line))

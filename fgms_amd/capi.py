@@ -17,7 +17,7 @@ SYMBOLS = [
     "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
-    "fgms_profile_reset", "fgms_probe_gather",
+    "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map",
 ]
 
 _lib = None
@@ -50,6 +50,9 @@ def lib():
                            i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_dgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_wgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_build_kernel_map.argtypes = [vp, i64, vp, i64, vp, i32, i32, i32, vp, vp, i64, vp, vp,
+                                        ctypes.POINTER(ctypes.c_int64), vp]
+    L.fgms_build_kernel_map.restype = i32
     L.fgms_probe_gather.argtypes = [vp, i32, i32, i32, vp, vp]
     L.fgms_probe_gather.restype = i32
     L.fgms_set_kernel_policy.argtypes = [i32]
@@ -215,6 +218,31 @@ def dgrad(out_grad, kernel, in_grad, kpos, in_map, out_map, plan=None):
         _p(out_grad), _p(kernel), _p(in_grad), _p(kpos), _p(in_map), _p(out_map),
         in_grad.shape[0], out_grad.shape[0], kernel.shape[1], kernel.shape[2], kernel.shape[0],
         in_map.numel(), _dtype(out_grad), _ph(plan), _stream()))
+
+
+def build_kernel_map(in_coords, out_coords, offsets, stride=1, skip_offset=None, capacity=None):
+    """Pair lists of a kernel map from int32 voxel coordinates on the device.
+    Returns (in_map, out_map, kernel_nnz, kpos): device int32 tensors, the maps trimmed
+    to the number of pairs found."""
+    import numpy as np
+    import torch
+    for t, n in ((in_coords, "in_coords"), (out_coords, "out_coords")):
+        if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous() or t.dim() != 2 or t.shape[1] != 3:
+            raise ValueError("%s must be a contiguous int32 [N, 3] tensor on the GPU" % n)
+    offs = np.ascontiguousarray(np.asarray(offsets, dtype=np.int32).reshape(-1, 3))
+    k_vol = len(offs)
+    n_in, n_out = in_coords.shape[0], out_coords.shape[0]
+    cap = k_vol * n_out if capacity is None else int(capacity)
+    in_map = torch.empty(max(cap, 1), dtype=torch.int32, device=in_coords.device)
+    out_map = torch.empty(max(cap, 1), dtype=torch.int32, device=in_coords.device)
+    knnz = torch.empty(k_vol, dtype=torch.int32, device=in_coords.device)
+    kpos = torch.empty(k_vol + 1, dtype=torch.int32, device=in_coords.device)
+    found = ctypes.c_int64(0)
+    _check(lib().fgms_build_kernel_map(
+        _p(in_coords), n_in, _p(out_coords), n_out, offs.ctypes.data_as(ctypes.c_void_p), k_vol,
+        int(stride), -1 if skip_offset is None else int(skip_offset), _p(in_map), _p(out_map), cap,
+        _p(knnz), _p(kpos), ctypes.byref(found), _stream()))
+    return in_map[:found.value], out_map[:found.value], knnz, kpos
 
 
 def probe_gather(feats, plan, for_dgrad=False):

@@ -79,6 +79,120 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *
   return FGMS_OK;
 }
 
+// ---- block pool: device memory of plans and of the map builder's temporaries --
+// hipMalloc / hipFree cost 50-100 us each and a plan needs a dozen blocks, which
+// made building a plan (once per kernel map, i.e. several times per training
+// step) three times as expensive as its kernels.  Freed blocks are kept per
+// device and handed out again to requests of similar size.  A block that may
+// still be read by queued work carries an event recorded on the stream that used
+// it last; whoever gets the block next makes its own stream wait for that event.
+namespace {
+struct PoolBlock {
+  void *ptr;
+  size_t bytes;
+  int device;
+  hipEvent_t ready;    // nullptr: idle
+};
+std::mutex g_pool_mutex;
+std::vector<PoolBlock> g_pool_free;
+std::map<void *, std::pair<size_t, int>> g_pool_live;   // ptr -> (bytes, device)
+size_t g_pool_cached = 0;
+constexpr size_t kPoolMaxCached = (size_t)2 << 30;
+}  // namespace
+
+int pool_alloc(void **ptr, size_t bytes, hipStream_t user) {
+  *ptr = nullptr;
+  if (bytes == 0) bytes = 256;
+  bytes = (bytes + 255) & ~(size_t)255;
+  int dev = 0;
+  FGMS_HIP_TRY(hipGetDevice(&dev));
+  PoolBlock got{};
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    int best = -1;
+    for (int i = 0; i < (int)g_pool_free.size(); ++i) {
+      const PoolBlock &b = g_pool_free[i];
+      if (b.device != dev || b.bytes < bytes || b.bytes > 2 * bytes + 4096) continue;
+      if (best < 0 || b.bytes < g_pool_free[best].bytes) best = i;
+    }
+    if (best >= 0) {
+      got = g_pool_free[best];
+      g_pool_free.erase(g_pool_free.begin() + best);
+      g_pool_cached -= got.bytes;
+      g_pool_live[got.ptr] = {got.bytes, dev};
+    }
+  }
+  if (got.ptr) {
+    if (got.ready) {
+      hipError_t e = hipStreamWaitEvent(user, got.ready, 0);
+      (void)hipEventDestroy(got.ready);
+      if (e != hipSuccess) {
+        set_error("pool_alloc: hipStreamWaitEvent: %s", hipGetErrorString(e));
+        return FGMS_E_HIP;
+      }
+    }
+    *ptr = got.ptr;
+    return FGMS_OK;
+  }
+  void *q = nullptr;
+  if (hipMalloc(&q, bytes) != hipSuccess) {
+    // give cached blocks back to the driver and try once more
+    pool_trim(0);
+    if (hipMalloc(&q, bytes) != hipSuccess) {
+      set_error("device allocation of %zu bytes failed", bytes);
+      return FGMS_E_NOMEM;
+    }
+  }
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  g_pool_live[q] = {bytes, dev};
+  *ptr = q;
+  return FGMS_OK;
+}
+
+void pool_free(void *ptr, hipStream_t last_user, bool idle) {
+  if (!ptr) return;
+  PoolBlock b{};
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_pool_live.find(ptr);
+    if (it == g_pool_live.end()) return;
+    b = PoolBlock{ptr, it->second.first, it->second.second, nullptr};
+    g_pool_live.erase(it);
+  }
+  if (!idle) {
+    // queued work may still read the block: mark the point after which it is free
+    hipEvent_t ev = nullptr;
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess ||
+        hipEventRecord(ev, last_user) != hipSuccess) {
+      if (ev) (void)hipEventDestroy(ev);
+      (void)hipFree(ptr);     // synchronises; also the path taken while the runtime shuts down
+      return;
+    }
+    b.ready = ev;
+  }
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  g_pool_free.push_back(b);
+  g_pool_cached += b.bytes;
+  while (g_pool_cached > kPoolMaxCached && !g_pool_free.empty()) {
+    PoolBlock old = g_pool_free.front();
+    g_pool_free.erase(g_pool_free.begin());
+    g_pool_cached -= old.bytes;
+    if (old.ready) (void)hipEventDestroy(old.ready);
+    (void)hipFree(old.ptr);
+  }
+}
+
+void pool_trim(size_t keep_bytes) {
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  while (g_pool_cached > keep_bytes && !g_pool_free.empty()) {
+    PoolBlock old = g_pool_free.front();
+    g_pool_free.erase(g_pool_free.begin());
+    g_pool_cached -= old.bytes;
+    if (old.ready) (void)hipEventDestroy(old.ready);
+    (void)hipFree(old.ptr);
+  }
+}
+
 // ---- profiling records -------------------------------------------------------
 namespace {
 struct ProfRec {
@@ -133,6 +247,7 @@ int check_common(const void *a, const void *b, const void *c, const int32_t *kpo
 }
 
 int run_gms(GmsArgs a, const Plan *plan) {
+  if (plan) plan->last_stream = a.stream;
   const bool dense = a.dense_k >= 0;
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
   if (g_policy != 1) {
@@ -145,6 +260,7 @@ int run_gms(GmsArgs a, const Plan *plan) {
 
 int run_wgrad(const WgradArgs &a) {
   if (a.n_pairs == 0) return FGMS_OK;
+  if (a.plan) a.plan->last_stream = a.stream;
   if (g_policy != 1 && mfma_wgrad_supported(a)) return launch_mfma_wgrad(a);
   return launch_generic_wgrad(a);
 }
@@ -319,6 +435,21 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
                     c_in, c_out, k_vol, n_pairs, dtype, plan, stream);
 }
 
+int fgms_build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords,
+                          int64_t n_out, const int32_t *offsets, int k_vol, int stride,
+                          int skip_offset, int32_t *in_map, int32_t *out_map, int64_t capacity,
+                          int32_t *kernel_nnz, int32_t *kpos, int64_t *n_pairs, void *stream) {
+  if (n_in < 0 || n_out < 0 || k_vol <= 0 || stride <= 0 || capacity < 0 || !offsets || !kernel_nnz ||
+      !kpos || !n_pairs || (n_in > 0 && !in_coords) || (n_out > 0 && !out_coords) ||
+      (capacity > 0 && (!in_map || !out_map)) || n_in > INT32_MAX ||
+      (int64_t)k_vol * n_out > INT32_MAX - 65536) {
+    set_error("fgms_build_kernel_map: bad argument");
+    return FGMS_E_INVALID;
+  }
+  return build_kernel_map(in_coords, n_in, out_coords, n_out, offsets, k_vol, stride, skip_offset,
+                          in_map, out_map, capacity, kernel_nnz, kpos, n_pairs, (hipStream_t)stream);
+}
+
 int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad, fgms_plan_t *plan,
                       void *stream) {
   const Plan *p = (const Plan *)plan;
@@ -326,6 +457,7 @@ int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad, fg
     set_error("fgms_probe_gather: bad argument");
     return FGMS_E_INVALID;
   }
+  p->last_stream = (hipStream_t)stream;
   void *sink = nullptr;
   int rc = workspace_get((hipStream_t)stream, 3, 256, &sink);
   if (rc) return rc;

@@ -86,6 +86,7 @@ struct Plan {
   int band_count;
   int32_t *band_start;   // [k_vol, band_count + 1]
   bool bands_ok;
+  mutable hipStream_t last_stream;   // the stream of the latest launch that read the plan
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -110,6 +111,12 @@ int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
 int launch_generic_gms(const GmsArgs &a);
 int launch_generic_wgrad(const WgradArgs &a);
 bool mfma_gms_supported(const GmsArgs &a);
+// Pooled device blocks (plans, map-builder temporaries).  `user`: the stream the
+// block will be used on; `last_user` / `idle`: the stream that used it last, or
+// idle = true when no queued work can still touch it.
+int pool_alloc(void **ptr, size_t bytes, hipStream_t user);
+void pool_free(void *ptr, hipStream_t last_user, bool idle);
+void pool_trim(size_t keep_bytes);
 int kernel_policy();   // fgms_set_kernel_policy's value
 int launch_mfma_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
@@ -118,6 +125,10 @@ bool small_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_small_gms(const GmsArgs &a, const Plan *p);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_planned_gms(const GmsArgs &a, const Plan *p);
+int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
+                     const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
+                     int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,
+                     int32_t *kpos, int64_t *n_pairs, hipStream_t stream);
 int launch_gather_probe(const Plan *p, const void *src, int c_src, int dtype, bool for_dgrad,
                         void *sink, hipStream_t stream);
 

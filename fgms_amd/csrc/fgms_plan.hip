@@ -159,10 +159,12 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->perm_out = p->perm_in = nullptr;
   p->band_count = 0; p->band_start = nullptr; p->bands_ok = false;
   p->fwd_ok = p->dgrad_ok = false;
+  p->last_stream = s;
   int *flags = nullptr;
   int rc = FGMS_OK;
+  bool synced = false;      // true once the stream has drained: freed blocks are idle then
   auto fail = [&](int code) {
-    if (flags) (void)hipFree(flags);
+    if (flags) pool_free(flags, s, synced);
     fgms_plan_destroy((fgms_plan_t *)p);
     return code;
   };
@@ -183,12 +185,12 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   const int band_rows = (int)((n_out + p->band_count - 1) / p->band_count);
   const size_t so = (size_t)n_out * k_vol, si = (size_t)n_in * k_vol;
   const size_t bo = (size_t)(n_out + 63) / 64, bi = (size_t)(n_in + 63) / 64;
-  if (hipMalloc((void **)&p->nbr_out, (so ? so : 1) * sizeof(int32_t)) != hipSuccess ||
-      hipMalloc((void **)&p->nbr_in, (si ? si : 1) * sizeof(int32_t)) != hipSuccess ||
-      hipMalloc((void **)&p->mask_out, (bo ? bo : 1) * sizeof(unsigned long long)) != hipSuccess ||
-      hipMalloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long)) != hipSuccess ||
-      hipMalloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t)) != hipSuccess ||
-      hipMalloc((void **)&flags, 4 * sizeof(int)) != hipSuccess) {
+  if (pool_alloc((void **)&p->nbr_out, (so ? so : 1) * sizeof(int32_t), s) != FGMS_OK ||
+      pool_alloc((void **)&p->nbr_in, (si ? si : 1) * sizeof(int32_t), s) != FGMS_OK ||
+      pool_alloc((void **)&p->mask_out, (bo ? bo : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
+      pool_alloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
+      pool_alloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), s) != FGMS_OK ||
+      pool_alloc((void **)&flags, 4 * sizeof(int), s) != FGMS_OK) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
   }
@@ -213,11 +215,11 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   std::vector<void *> tmp_more;
   auto free_tmp = [&]() {
     for (int d = 0; d < 2; ++d) {
-      if (tmp_tab[d]) (void)hipFree(tmp_tab[d]);
-      if (tmp_mask[d]) (void)hipFree(tmp_mask[d]);
+      if (tmp_tab[d]) pool_free(tmp_tab[d], s, synced);
+      if (tmp_mask[d]) pool_free(tmp_mask[d], s, synced);
       tmp_tab[d] = nullptr; tmp_mask[d] = nullptr;
     }
-    for (void *q : tmp_more) (void)hipFree(q);
+    for (void *q : tmp_more) pool_free(q, s, synced);
     tmp_more.clear();
   };
   static const bool sort_rows = !(getenv("FGMS_PLAN_SORT") && atoi(getenv("FGMS_PLAN_SORT")) == 0);
@@ -231,10 +233,10 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       if (n == 0) continue;
       if (sort_rows && n > 64) {
         int32_t *sorted = nullptr;
-        if (hipMalloc((void **)&tmp_mask[d], (size_t)n * sizeof(unsigned long long)) != hipSuccess ||
-            hipMalloc((void **)&perm, (size_t)n * sizeof(int32_t)) != hipSuccess ||
-            hipMalloc((void **)&sorted, (size_t)n * k_vol * sizeof(int32_t)) != hipSuccess) {
-          if (sorted) (void)hipFree(sorted);
+        if (pool_alloc((void **)&tmp_mask[d], (size_t)n * sizeof(unsigned long long), s) != FGMS_OK ||
+            pool_alloc((void **)&perm, (size_t)n * sizeof(int32_t), s) != FGMS_OK ||
+            pool_alloc((void **)&sorted, (size_t)n * k_vol * sizeof(int32_t), s) != FGMS_OK) {
+          if (sorted) pool_free(sorted, s, synced);
           free_tmp();
           set_error("fgms_plan_create: reorder allocation failed");
           return fail(FGMS_E_NOMEM);
@@ -245,13 +247,13 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
         int32_t *rows_in = nullptr;
         void *sort_tmp = nullptr;
         size_t sort_bytes = 0;
-        bool ok = hipMalloc((void **)&keys_out, (size_t)n * sizeof(unsigned long long)) == hipSuccess;
+        bool ok = pool_alloc((void **)&keys_out, (size_t)n * sizeof(unsigned long long), s) == FGMS_OK;
         if (ok) tmp_more.push_back(keys_out);
-        ok = ok && hipMalloc((void **)&rows_in, (size_t)n * sizeof(int32_t)) == hipSuccess;
+        ok = ok && pool_alloc((void **)&rows_in, (size_t)n * sizeof(int32_t), s) == FGMS_OK;
         if (ok) tmp_more.push_back(rows_in);
         ok = ok && rocprim::radix_sort_pairs(nullptr, sort_bytes, tmp_mask[d], keys_out, rows_in, perm,
                                              (size_t)n, 0u, (unsigned)k_vol, s) == hipSuccess;
-        ok = ok && hipMalloc(&sort_tmp, sort_bytes ? sort_bytes : 1) == hipSuccess;
+        ok = ok && pool_alloc(&sort_tmp, sort_bytes, s) == FGMS_OK;
         if (ok) tmp_more.push_back(sort_tmp);
         if (ok) {
           iota_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(rows_in, (int)n);
@@ -259,7 +261,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
                                          (size_t)n, 0u, (unsigned)k_vol, s) == hipSuccess;
         }
         if (!ok) {
-          (void)hipFree(sorted);
+          pool_free(sorted, s, synced);
           free_tmp();
           set_error("fgms_plan_create: row sort failed");
           return fail(FGMS_E_HIP);
@@ -283,8 +285,9 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
     set_error("fgms_plan_create: reading the build flags failed");
     return fail(FGMS_E_HIP);
   }
+  synced = true;
   free_tmp();
-  (void)hipFree(flags);
+  pool_free(flags, s, synced);
   flags = nullptr;
   if (h[0]) {
     set_error("fgms_plan_create: a map index is outside [0, n_in) x [0, n_out)");
@@ -300,13 +303,13 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
 void fgms_plan_destroy(fgms_plan_t *plan) {
   Plan *p = (Plan *)plan;
   if (!p) return;
-  if (p->nbr_out) (void)hipFree(p->nbr_out);
-  if (p->nbr_in) (void)hipFree(p->nbr_in);
-  if (p->mask_out) (void)hipFree(p->mask_out);
-  if (p->mask_in) (void)hipFree(p->mask_in);
-  if (p->perm_out) (void)hipFree(p->perm_out);
-  if (p->perm_in) (void)hipFree(p->perm_in);
-  if (p->band_start) (void)hipFree(p->band_start);
+  if (p->nbr_out) pool_free(p->nbr_out, p->last_stream, false);
+  if (p->nbr_in) pool_free(p->nbr_in, p->last_stream, false);
+  if (p->mask_out) pool_free(p->mask_out, p->last_stream, false);
+  if (p->mask_in) pool_free(p->mask_in, p->last_stream, false);
+  if (p->perm_out) pool_free(p->perm_out, p->last_stream, false);
+  if (p->perm_in) pool_free(p->perm_in, p->last_stream, false);
+  if (p->band_start) pool_free(p->band_start, p->last_stream, false);
   delete p;
 }
 

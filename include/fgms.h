@@ -137,6 +137,28 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
 void fgms_set_kernel_policy(int policy);
 
 /*
+ * Kernel-map builder.  No counterpart in the reference, whose scripts load the
+ * maps from files (cpu-check.py:89-94, spconv-test.py:64-73); this is the step
+ * right before the path.  Finds every pair (i, o) with
+ *     in_coords[i] == out_coords[o] * stride + offsets[k]
+ * and writes them grouped by offset k, ascending o inside an offset (if input
+ * rows share a coordinate the smallest row index is taken):
+ * in_map / out_map (device, room for `capacity` pairs; k_vol * n_out always
+ * suffices), kernel_nnz[k_vol] and kpos[k_vol + 1] (device), *n_pairs (host).
+ * in_coords / out_coords: device int32 [n][3], every component in
+ * [-2^20, 2^20); offsets: HOST int32 [k_vol][3]; skip_offset: an offset to
+ * leave empty (the centre, for callers that use separate_mid), or -1.
+ * Synchronises the stream once.  FGMS_E_INVALID if a coordinate is out of
+ * range or the pairs do not fit `capacity` (*n_pairs is set, the lists hold
+ * the first `capacity` pairs).
+ */
+int fgms_build_kernel_map(const int32_t *in_coords, int64_t n_in,
+                          const int32_t *out_coords, int64_t n_out,
+                          const int32_t *offsets, int k_vol, int stride, int skip_offset,
+                          int32_t *in_map, int32_t *out_map, int64_t capacity,
+                          int32_t *kernel_nnz, int32_t *kpos, int64_t *n_pairs, void *stream);
+
+/*
  * Diagnostic, no counterpart in the reference: reads exactly the feature rows
  * the output-stationary forward (for_dgrad = 0: feats = in_feats, c_src = c_in)
  * or input-gradient kernel (for_dgrad != 0: feats = out_feats_grad,
