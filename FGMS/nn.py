@@ -40,6 +40,14 @@ class KernelMap:
         self.qkpos, self.qsum = kpos_quantized(kn, self.kpos, self.k_vol, _Q)
         self.n_in, self.n_out = int(n_in), int(n_out)
 
+    @classmethod
+    def from_coords(cls, in_coords, out_coords, offsets, stride=1):
+        """Builds the map on the device from int32 voxel coordinates ``[N, 3]``: pairs
+        (i, o) with ``in_coords[i] == out_coords[o] * stride + offsets[k]``."""
+        from fgms_amd import capi
+        in_map, out_map, knnz, _ = capi.build_kernel_map(in_coords, out_coords, offsets, stride)
+        return cls(in_map, out_map, knnz, in_coords.shape[0], out_coords.shape[0])
+
     def transposed(self):
         """The map of the transposed convolution: the same pairs, roles swapped."""
         return KernelMap(self.out_map, self.in_map, self.kernel_nnz, self.n_out, self.n_in)

@@ -80,6 +80,20 @@ def test_module_trains():
     assert backend.fgms_plan_cache_size() >= 1
 
 
+def test_kernel_map_from_coordinates():
+    from FGMS import nn as fnn
+    rng = np.random.default_rng(43)
+    vox = clouds.dedup(clouds._sphere_shell(rng, np.array([12., 12, 12]), 7.0, 2500), 24)
+    want = clouds.build_kernel_map(vox, vox, clouds.offsets_cube(3))
+    kmap = fnn.KernelMap.from_coords(torch.from_numpy(vox).cuda(), torch.from_numpy(vox).cuda(),
+                                     clouds.offsets_cube(3))
+    assert np.array_equal(kmap.in_map.cpu().numpy(), want[0])
+    assert np.array_equal(kmap.out_map.cpu().numpy(), want[1])
+    assert np.array_equal(kmap.kernel_nnz.numpy(), want[2])
+    y = fnn.sparse_conv(torch.randn(len(vox), 32, device="cuda"), torch.randn(27, 32, 32, device="cuda"), kmap)
+    assert y.shape == (len(vox), 32) and torch.isfinite(y).all()
+
+
 def test_kernel_map_checks_its_sizes():
     from FGMS import nn as fnn
     e = torch.zeros(5, dtype=torch.int32, device="cuda")
