@@ -86,6 +86,12 @@ struct Plan {
   int band_count;
   int32_t *band_start;   // [k_vol, band_count + 1]
   bool bands_ok;
+  // Workgroup -> tile of 256 positions for the output-stationary kernel:
+  // workgroup b runs on XCD b % 8 and takes tile tile_out[b] (or -1: none), chosen
+  // so that a tile runs on the XCD that owns the eighth of the cloud most of its
+  // rows lie in (their neighbours then meet in that XCD's L2).  nullptr: tile = b.
+  int32_t *tile_out, *tile_in;
+  int tile_grid_out, tile_grid_in;   // entries of the tables (a multiple of 8)
   mutable hipStream_t last_stream;   // the stream of the latest launch that read the plan
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row

@@ -435,7 +435,8 @@ template <typename T, int NT, int S>
 __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
-    const int32_t *__restrict__ perm, int n_dst, int k_vol, int c_src, int c_dst) {
+    const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
+    int c_src, int c_dst) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
   constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
@@ -454,7 +455,9 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   const int4v *packed4 = reinterpret_cast<const int4v *>(packed);
   const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
 
-  const int row0 = blockIdx.x * kTileRows + wave * kWaveRows;
+  const int tile = tile_order ? tile_order[blockIdx.x] : (int)blockIdx.x;
+  if (tile < 0) return;
+  const int row0 = tile * kTileRows + wave * kWaveRows;
   const int my_row = row0 + lane;
   const bool in_range = my_row < n_dst;
   didx[lane] = in_range ? (perm ? perm[my_row] : my_row) : -1;   // my_row is a position in the plan's row order
@@ -630,11 +633,12 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
 
 template <typename T, int NT, int S>
 int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
-                const unsigned long long *masks, const int32_t *perm) {
+                const unsigned long long *masks, const int32_t *perm, const int32_t *tile_order,
+                int tile_grid) {
   const T *packed = nullptr;
   int rc = pack_weights<T>(a, s, &packed);
   if (rc != FGMS_OK) return rc;
-  const unsigned gx = (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
+  const unsigned gx = tile_order ? (unsigned)tile_grid : (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
   if (gx == 0) return FGMS_OK;
   auto kern = gms_rows_kernel<T, NT, S>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -643,8 +647,8 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   {
     ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
     kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_rows_bytes, a.stream>>>(
-        (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, (int)a.n_dst, a.k_vol, s.c_src,
-        s.c_dst);
+        (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
+        s.c_src, s.c_dst);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -742,12 +746,14 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p) {
   const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
   const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
   const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
+  const int32_t *tile_order = a.transpose_w ? p->tile_in : p->tile_out;
+  const int tile_grid = a.transpose_w ? p->tile_grid_in : p->tile_grid_out;
   if (a.dtype == FGMS_F16)
     return dispatch_rows_shape<__half>(s, [&](auto nt, auto sv) {
-      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm);
+      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm, tile_order, tile_grid);
     });
   return dispatch_rows_shape<float>(s, [&](auto nt, auto sv) {
-    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm);
+    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm, tile_order, tile_grid);
   });
 }
 

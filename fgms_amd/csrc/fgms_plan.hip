@@ -108,6 +108,39 @@ __global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32
   }
 }
 
+// One thread per XCD.  A tile's home XCD is the eighth of the cloud its middle row
+// lies in (original row numbers follow the voxel order, i.e. space).  Every XCD
+// first takes its own tiles, in order, up to cap = ceil(tiles / 8); what does not
+// fit is dealt, after a barrier, to the XCDs that still have room.
+// order[pos * 8 + xcd] = tile, -1 where a list ends early.
+__global__ void tile_homes_kernel(const int32_t *__restrict__ perm, int n_rows, int n_tiles, int cap,
+                                  int32_t *__restrict__ order) {
+  __shared__ int filled[8];
+  __shared__ int spill_count;
+  extern __shared__ int32_t spill[];            // [n_tiles]
+  const int x = threadIdx.x;
+  if (x == 0) spill_count = 0;
+  __syncthreads();
+  if (x < 8) {
+    int mine = 0;
+    for (int t = 0; t < n_tiles; ++t) {
+      const int mid = min(t * 256 + 128, n_rows - 1);
+      const int home = (int)((long long)(perm ? perm[mid] : mid) * 8 / n_rows);
+      if (home != x) continue;
+      if (mine < cap) order[mine++ * 8 + x] = t;
+      else spill[atomicAdd(&spill_count, 1)] = t;
+    }
+    filled[x] = mine;
+  }
+  __syncthreads();
+  if (x == 0) {
+    int next = 0;
+    for (int q = 0; q < 8; ++q)
+      for (int pos = filled[q]; pos < cap; ++pos)
+        order[pos * 8 + q] = next < spill_count ? spill[next++] : -1;
+  }
+}
+
 __global__ void iota_kernel(int32_t *__restrict__ p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = i;
@@ -158,6 +191,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->nbr_out = p->nbr_in = nullptr; p->mask_out = p->mask_in = nullptr;
   p->perm_out = p->perm_in = nullptr;
   p->band_count = 0; p->band_start = nullptr; p->bands_ok = false;
+  p->tile_out = p->tile_in = nullptr; p->tile_grid_out = p->tile_grid_in = 0;
   p->fwd_ok = p->dgrad_ok = false;
   p->last_stream = s;
   int *flags = nullptr;
@@ -271,6 +305,19 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
         tab = sorted;
       }
       block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask);
+      // tile -> XCD homes pay off once every XCD has a few dozen tiles of its own
+      static const bool xcd_homes = !(getenv("FGMS_XCD_HOME") && atoi(getenv("FGMS_XCD_HOME")) == 0);
+      const int n_tiles = (int)((n + 255) / 256);
+      if (xcd_homes && n_tiles >= 256 && (size_t)n_tiles * sizeof(int32_t) <= 60000) {
+        int32_t *&order = d ? p->tile_in : p->tile_out;
+        const int cap = (n_tiles + 7) / 8;
+        if (pool_alloc((void **)&order, (size_t)cap * 8 * sizeof(int32_t), s) != FGMS_OK) {
+          free_tmp();
+          return fail(FGMS_E_NOMEM);
+        }
+        (d ? p->tile_grid_in : p->tile_grid_out) = cap * 8;
+        tile_homes_kernel<<<1, 64, (size_t)n_tiles * sizeof(int32_t), s>>>(perm, (int)n, n_tiles, cap, order);
+      }
     }
     if (hipGetLastError() != hipSuccess) {
       free_tmp();
@@ -310,6 +357,8 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->perm_out) pool_free(p->perm_out, p->last_stream, false);
   if (p->perm_in) pool_free(p->perm_in, p->last_stream, false);
   if (p->band_start) pool_free(p->band_start, p->last_stream, false);
+  if (p->tile_out) pool_free(p->tile_out, p->last_stream, false);
+  if (p->tile_in) pool_free(p->tile_in, p->last_stream, false);
   delete p;
 }
 
