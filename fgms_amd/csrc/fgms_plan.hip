@@ -108,36 +108,74 @@ __global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32
   }
 }
 
-// One thread per XCD.  A tile's home XCD is the eighth of the cloud its middle row
-// lies in (original row numbers follow the voxel order, i.e. space).  Every XCD
-// first takes its own tiles, in order, up to cap = ceil(tiles / 8); what does not
-// fit is dealt, after a barrier, to the XCDs that still have room.
-// order[pos * 8 + xcd] = tile, -1 where a list ends early.
-__global__ void tile_homes_kernel(const int32_t *__restrict__ perm, int n_rows, int n_tiles, int cap,
-                                  int32_t *__restrict__ order) {
-  __shared__ int filled[8];
-  __shared__ int spill_count;
+// A tile's home XCD is the eighth of the cloud its middle row lies in (original
+// row numbers follow the voxel order, i.e. space).  Every XCD takes its own tiles,
+// in tile order, up to cap = ceil(tiles / 8); what does not fit is dealt, in tile
+// order as well, to the XCDs that still have room.  order[pos * 8 + xcd] = tile;
+// the table is pre-filled with -1 for lists that end early.  One workgroup of
+// 1024 threads, 1024 tiles per round; ranks come from wave ballots and a prefix
+// over the 16 waves, so the result does not depend on timing.
+__global__ __launch_bounds__(1024) void tile_homes_kernel(const int32_t *__restrict__ perm, int n_rows,
+                                                          int n_tiles, int cap,
+                                                          int32_t *__restrict__ order) {
+  constexpr int kWavesHere = 16, kClasses = 9;   // 8 homes + "does not fit"
+  __shared__ int wave_cnt[kWavesHere][kClasses];
+  __shared__ int run[kClasses];
   extern __shared__ int32_t spill[];            // [n_tiles]
-  const int x = threadIdx.x;
-  if (x == 0) spill_count = 0;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const unsigned long long below = (1ull << lane) - 1;
+  if (tid < kClasses) run[tid] = 0;
   __syncthreads();
-  if (x < 8) {
-    int mine = 0;
-    for (int t = 0; t < n_tiles; ++t) {
+  for (int base = 0; base < n_tiles; base += 1024) {
+    const int t = base + tid;
+    int home = -1;
+    if (t < n_tiles) {
       const int mid = min(t * 256 + 128, n_rows - 1);
-      const int home = (int)((long long)(perm ? perm[mid] : mid) * 8 / n_rows);
-      if (home != x) continue;
-      if (mine < cap) order[mine++ * 8 + x] = t;
-      else spill[atomicAdd(&spill_count, 1)] = t;
+      home = (int)((long long)(perm ? perm[mid] : mid) * 8 / n_rows);
     }
-    filled[x] = mine;
+    int in_wave = 0;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const unsigned long long b = __ballot(home == x);
+      if (lane == 0) wave_cnt[wave][x] = __builtin_popcountll(b);
+      if (home == x) in_wave = __builtin_popcountll(b & below);
+    }
+    __syncthreads();
+    int rank = -1;
+    if (home >= 0) {
+      rank = run[home] + in_wave;
+      for (int w = 0; w < wave; ++w) rank += wave_cnt[w][home];
+    }
+    const bool fits = home >= 0 && rank < cap;
+    if (fits) order[rank * 8 + home] = t;
+    const bool spilled = home >= 0 && !fits;
+    const unsigned long long sb = __ballot(spilled);
+    if (lane == 0) wave_cnt[wave][8] = __builtin_popcountll(sb);
+    __syncthreads();
+    if (spilled) {
+      int pos = run[8] + __builtin_popcountll(sb & below);
+      for (int w = 0; w < wave; ++w) pos += wave_cnt[w][8];
+      spill[pos] = t;
+    }
+    __syncthreads();
+    if (tid < kClasses) {
+      int add = 0;
+      for (int w = 0; w < kWavesHere; ++w) add += wave_cnt[w][tid];
+      run[tid] += add;
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  if (x == 0) {
-    int next = 0;
-    for (int q = 0; q < 8; ++q)
-      for (int pos = filled[q]; pos < cap; ++pos)
-        order[pos * 8 + q] = next < spill_count ? spill[next++] : -1;
+  const int n_spill = run[8];
+  for (int sidx = tid; sidx < n_spill; sidx += 1024) {
+    int left = sidx;
+    for (int q = 0; q < 8; ++q) {
+      const int filled = min(run[q], cap), room = cap - filled;
+      if (left < room) {
+        order[(filled + left) * 8 + q] = spill[sidx];
+        break;
+      }
+      left -= room;
+    }
   }
 }
 
@@ -316,7 +354,11 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
           return fail(FGMS_E_NOMEM);
         }
         (d ? p->tile_grid_in : p->tile_grid_out) = cap * 8;
-        tile_homes_kernel<<<1, 64, (size_t)n_tiles * sizeof(int32_t), s>>>(perm, (int)n, n_tiles, cap, order);
+        if ((rc = fill_i32(order, (size_t)cap * 8, -1, s))) {
+          free_tmp();
+          return fail(rc);
+        }
+        tile_homes_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), s>>>(perm, (int)n, n_tiles, cap, order);
       }
     }
     if (hipGetLastError() != hipSuccess) {
