@@ -258,14 +258,15 @@ __device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__rest
 // columns of one row and a destination row is read and written as whole
 // 64..256-byte runs by neighbouring lanes instead of 4 bytes per lane.
 // stage: the wave's staging tile, 64 * 2*S * 16 bytes.
-template <typename T, int NT, int S>
+template <typename T, int NT, int S, bool ATOMIC>
 __device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__restrict__ dst,
                                              const int *__restrict__ rows, float *__restrict__ stage,
                                              int c_dst, int cd0, int lane) {
   constexpr int COLS = NT * 32;
   constexpr int R = (64 * 2 * S * 16) / (COLS * 4) >= 32 ? 32 : (64 * 2 * S * 16) / (COLS * 4);
   if constexpr (R < 8) {
-    add_rows<T, NT>(acc, dst, rows, c_dst, cd0, lane);
+    if constexpr (ATOMIC) write_tile<T, NT, true>(acc, dst, rows, c_dst, cd0, lane);
+    else add_rows<T, NT>(acc, dst, rows, c_dst, cd0, lane);
   } else {
     constexpr int CH = COLS / 4;            // 16-byte chunks per staged row
     constexpr int IT = R * CH / 64;         // chunks per lane and pass
@@ -289,7 +290,21 @@ __device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__
         part[it] = *reinterpret_cast<const float4v *>(stage + (e / CH) * COLS + (e % CH) * 4);
         row[it] = rows[p * R + e / CH];
       }
-      if constexpr (sizeof(T) == 4) {
+      if constexpr (ATOMIC) {
+        // another workgroup adds its share of the offsets to the same rows
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+          if (row[it] < 0) continue;
+          T *p = dst + (size_t)row[it] * c_dst + cd0 + ((it * 64 + lane) % CH) * 4;
+          if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) atomic_add(reinterpret_cast<float *>(p) + q, part[it][q]);
+          } else {
+            atomic_add_pk(reinterpret_cast<__half *>(p), part[it][0], part[it][1]);
+            atomic_add_pk(reinterpret_cast<__half *>(p) + 2, part[it][2], part[it][3]);
+          }
+        }
+      } else if constexpr (sizeof(T) == 4) {
         float4v old[IT];
 #pragma unroll
         for (int it = 0; it < IT; ++it)
@@ -436,7 +451,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
-    int c_src, int c_dst) {
+    int c_src, int c_dst, int part_stages) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
   constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
@@ -470,6 +485,27 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   __syncthreads();
   unsigned long long todo = wg_mask;
   if (!todo) return;
+  // gridDim.z > 1: a tile is shared by up to gridDim.z workgroups, each takes a run
+  // of the tile's offsets and adds its partial result with atomics.
+  bool shared_tile = false;
+  if (gridDim.z > 1) {
+    const int n_off = __builtin_popcountll(todo);
+    const int want = (n_off * slabs + part_stages - 1) / part_stages;
+    const int parts = min((int)gridDim.z, max(want, 1));
+    if ((int)blockIdx.z >= parts) return;
+    if (parts > 1) {
+      shared_tile = true;
+      const int per = (n_off + parts - 1) / parts;
+      for (int i = 0; i < (int)blockIdx.z * per; ++i) todo &= todo - 1;      // offsets of earlier parts
+      unsigned long long mine = 0, rest = todo;
+      for (int i = 0; i < per && rest; ++i) {
+        mine |= rest & (0 - rest);
+        rest &= rest - 1;
+      }
+      todo = mine;
+      if (!todo) return;
+    }
+  }
 
   float16v acc[2][NT];
 #pragma unroll
@@ -550,7 +586,10 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   }
   if (wave_mask) {
     wave_lds_fence();
-    add_rows_lds<T, NT, S>(acc, dst, didx, reinterpret_cast<float *>(a_lds), c_dst, nt0 * 32, lane);
+    if (shared_tile)
+      add_rows_lds<T, NT, S, true>(acc, dst, didx, reinterpret_cast<float *>(a_lds), c_dst, nt0 * 32, lane);
+    else
+      add_rows_lds<T, NT, S, false>(acc, dst, didx, reinterpret_cast<float *>(a_lds), c_dst, nt0 * 32, lane);
   }
 }
 
@@ -644,11 +683,25 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)s.lds_rows_bytes));
+  // A launch that fills less than half of the chip's workgroup slots shares every
+  // tile between two workgroups, each taking half of the tile's offsets and adding
+  // its part with atomics: twice the workgroups, half the critical path.  (Two
+  // parts only: the sum of two partial results does not depend on their order.
+  // On launches that fill the chip the atomics cost more than the split gains.)
+  const int slabs = s.c_src / (2 * S * s.E);
+  const unsigned gy = (unsigned)(s.c_dst / (32 * NT));
+  const int64_t slots = (int64_t)num_cus() * (NT == 4 ? 2 : 3);
+  int part_stages = 0;
+  unsigned gz = 1;
+  if ((int64_t)gx * gy * 2 <= slots && a.k_vol * slabs >= 8) {
+    part_stages = (a.k_vol * slabs + 1) / 2;
+    gz = 2;
+  }
   {
     ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
-    kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_rows_bytes, a.stream>>>(
+    kern<<<dim3(gx, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
-        s.c_src, s.c_dst);
+        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
