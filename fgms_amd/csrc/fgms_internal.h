@@ -124,6 +124,7 @@ int pool_alloc(void **ptr, size_t bytes, hipStream_t user);
 void pool_free(void *ptr, hipStream_t last_user, bool idle);
 void pool_trim(size_t keep_bytes);
 int kernel_policy();   // fgms_set_kernel_policy's value
+int num_cus();         // compute units of the current device
 int launch_mfma_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);

@@ -485,6 +485,14 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   __syncthreads();
   unsigned long long todo = wg_mask;
   if (!todo) return;
+  // The launch lasts as long as its longest tile, and the tiles with the longest
+  // offset lists are few: they get the instruction issue priority, so that they run
+  // at their own pace while the many short tiles share what is left.
+  {
+    const int n_off = __builtin_popcountll(todo);
+    if (n_off * 4 > k_vol * 3) __builtin_amdgcn_s_setprio(3);
+    else if (n_off * 2 > k_vol) __builtin_amdgcn_s_setprio(1);
+  }
   // gridDim.z > 1: a tile is shared by up to gridDim.z workgroups, each takes a run
   // of the tile's offsets and adds its partial result with atomics.
   bool shared_tile = false;

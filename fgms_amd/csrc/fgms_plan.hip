@@ -108,70 +108,81 @@ __global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32
   }
 }
 
-// A tile's home XCD is the eighth of the cloud its middle row lies in (original
-// row numbers follow the voxel order, i.e. space).  Every XCD takes its own tiles,
-// in tile order, up to cap = ceil(tiles / 8); what does not fit is dealt, in tile
-// order as well, to the XCDs that still have room.  order[pos * 8 + xcd] = tile;
-// the table is pre-filled with -1 for lists that end early.  One workgroup of
-// 1024 threads, 1024 tiles per round; ranks come from wave ballots and a prefix
-// over the 16 waves, so the result does not depend on timing.
-__global__ __launch_bounds__(1024) void tile_homes_kernel(const int32_t *__restrict__ perm, int n_rows,
-                                                          int n_tiles, int cap,
-                                                          int32_t *__restrict__ order) {
-  constexpr int kWavesHere = 16, kClasses = 9;   // 8 homes + "does not fit"
-  __shared__ int wave_cnt[kWavesHere][kClasses];
-  __shared__ int run[kClasses];
-  extern __shared__ int32_t spill[];            // [n_tiles]
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const unsigned long long below = (1ull << lane) - 1;
-  if (tid < kClasses) run[tid] = 0;
-  __syncthreads();
-  for (int base = 0; base < n_tiles; base += 1024) {
-    const int t = base + tid;
-    int home = -1;
-    if (t < n_tiles) {
-      const int mid = min(t * 256 + 128, n_rows - 1);
-      home = (int)((long long)(perm ? perm[mid] : mid) * 8 / n_rows);
-    }
-    int in_wave = 0;
-#pragma unroll
-    for (int x = 0; x < 8; ++x) {
-      const unsigned long long b = __ballot(home == x);
-      if (lane == 0) wave_cnt[wave][x] = __builtin_popcountll(b);
-      if (home == x) in_wave = __builtin_popcountll(b & below);
-    }
-    __syncthreads();
-    int rank = -1;
-    if (home >= 0) {
-      rank = run[home] + in_wave;
-      for (int w = 0; w < wave; ++w) rank += wave_cnt[w][home];
-    }
-    const bool fits = home >= 0 && rank < cap;
-    if (fits) order[rank * 8 + home] = t;
-    const bool spilled = home >= 0 && !fits;
-    const unsigned long long sb = __ballot(spilled);
-    if (lane == 0) wave_cnt[wave][8] = __builtin_popcountll(sb);
-    __syncthreads();
-    if (spilled) {
-      int pos = run[8] + __builtin_popcountll(sb & below);
-      for (int w = 0; w < wave; ++w) pos += wave_cnt[w][8];
-      spill[pos] = t;
-    }
-    __syncthreads();
-    if (tid < kClasses) {
-      int add = 0;
-      for (int w = 0; w < kWavesHere; ++w) add += wave_cnt[w][tid];
-      run[tid] += add;
-    }
-    __syncthreads();
+// Dispatch order of the 256-position tiles of the output-stationary kernel.
+// Workgroup b runs on XCD b % 8 and, inside an XCD, workgroup number q = b / 8
+// lands on CU q % cus_per_xcd (the dispatcher goes round the CUs).
+//  * A tile's home XCD is the eighth of the cloud its middle row lies in
+//    (original row numbers follow the voxel order, i.e. space), so that
+//    neighbouring rows meet in one L2.
+//  * Inside an XCD the tiles are ranked by the number of offsets they use, most
+//    first: the launch lasts as long as its longest tile, so those must start
+//    first.  Ranks are laid over the CUs in a snake (round 0 forwards, round 1
+//    backwards, ...), so every CU gets a mix of long and short tiles instead of
+//    three long ones competing for the same SIMDs.
+//  * Every XCD takes at most cap = ceil(tiles / 8) tiles; the lightest tiles of an
+//    overfull XCD go to the XCDs that have room.
+// order[q * 8 + xcd] = tile (pre-filled with -1).  One workgroup; which of two
+// equally heavy tiles comes first depends on timing, the results do not.
+__global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restrict__ perm,
+                                                          const unsigned long long *__restrict__ block_masks,
+                                                          int n_rows, int n_tiles, int cap,
+                                                          int cus_per_xcd, int32_t *__restrict__ order) {
+  constexpr int kPc = 65;                         // popcount classes 0..64
+  __shared__ int hist[8][kPc];                    // tiles per (home, popcount), then start ranks
+  __shared__ int cursor[8][kPc];
+  __shared__ int total[8];
+  __shared__ int spill_count;
+  extern __shared__ int32_t spill[];              // [n_tiles]
+  const int tid = threadIdx.x;
+  const int n_blocks = (n_rows + 63) / 64;
+  for (int i = tid; i < 8 * kPc; i += 1024) {
+    (&hist[0][0])[i] = 0;
+    (&cursor[0][0])[i] = 0;
   }
-  const int n_spill = run[8];
-  for (int sidx = tid; sidx < n_spill; sidx += 1024) {
+  if (tid == 0) spill_count = 0;
+  __syncthreads();
+  auto classify = [&](int t, int &home, int &pc) {
+    const int mid = min(t * 256 + 128, n_rows - 1);
+    home = (int)((long long)(perm ? perm[mid] : mid) * 8 / n_rows);
+    unsigned long long m = 0;
+    for (int b = 4 * t; b < min(4 * t + 4, n_blocks); ++b) m |= block_masks[b];
+    pc = __builtin_popcountll(m);
+  };
+  for (int t = tid; t < n_tiles; t += 1024) {
+    int home, pc;
+    classify(t, home, pc);
+    atomicAdd(&hist[home][pc], 1);
+  }
+  __syncthreads();
+  if (tid < 8) {                                  // start rank of each class, heaviest first
+    int run = 0;
+    for (int pc = kPc - 1; pc >= 0; --pc) {
+      const int n = hist[tid][pc];
+      hist[tid][pc] = run;
+      run += n;
+    }
+    total[tid] = run;
+  }
+  __syncthreads();
+  auto position = [&](int rank) {                 // snake over the CUs
+    const int round = rank / cus_per_xcd, j = rank % cus_per_xcd;
+    const int in_round = min(cus_per_xcd, cap - round * cus_per_xcd);
+    return round * cus_per_xcd + ((round & 1) ? in_round - 1 - j : j);
+  };
+  for (int t = tid; t < n_tiles; t += 1024) {
+    int home, pc;
+    classify(t, home, pc);
+    const int rank = hist[home][pc] + atomicAdd(&cursor[home][pc], 1);
+    if (rank < cap) order[position(rank) * 8 + home] = t;
+    else spill[atomicAdd(&spill_count, 1)] = t;
+  }
+  __syncthreads();
+  for (int sidx = tid; sidx < spill_count; sidx += 1024) {
     int left = sidx;
     for (int q = 0; q < 8; ++q) {
-      const int filled = min(run[q], cap), room = cap - filled;
+      const int filled = min(total[q], cap), room = cap - filled;
       if (left < room) {
-        order[(filled + left) * 8 + q] = spill[sidx];
+        order[position(filled + left) * 8 + q] = spill[sidx];
         break;
       }
       left -= room;
@@ -358,7 +369,8 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
           free_tmp();
           return fail(rc);
         }
-        tile_homes_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), s>>>(perm, (int)n, n_tiles, cap, order);
+        tile_order_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), s>>>(
+            perm, mask, (int)n, n_tiles, cap, num_cus() >= 8 ? num_cus() / 8 : 1, order);
       }
     }
     if (hipGetLastError() != hipSuccess) {
