@@ -190,6 +190,34 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restr
   }
 }
 
+// cells[q * 8 + xcd]: the q-th cell of XCD xcd, cell = offset * 65536 + band.  XCD x
+// owns the bands x, x + 8, ...; its cells are ranked by pair count, most first (the
+// launch ends with its longest workgroup, so those start first), ties by cell
+// number, and the ranks are laid over the CUs in a snake like the tiles above.
+// One thread per cell; a cell's rank is found by comparing with the other cells of
+// its XCD (a few hundred).
+__global__ void band_cells_kernel(const int32_t *__restrict__ band_start, int k_vol, int bands,
+                                  int cus_per_xcd, int32_t *__restrict__ cells) {
+  const int per_xcd = (bands / 8) * k_vol;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;   // cell number inside its XCD: (band / 8) * k_vol + k
+  const int x = blockIdx.y;
+  if (c >= per_xcd) return;
+  auto pairs_of = [&](int cell) {
+    const int k = cell % k_vol, band = (cell / k_vol) * 8 + x;
+    return band_start[k * (bands + 1) + band + 1] - band_start[k * (bands + 1) + band];
+  };
+  const int mine = pairs_of(c);
+  int rank = 0;
+  for (int o = 0; o < per_xcd; ++o) {
+    const int theirs = pairs_of(o);
+    rank += (theirs > mine || (theirs == mine && o < c)) ? 1 : 0;
+  }
+  const int round = rank / cus_per_xcd, j = rank % cus_per_xcd;
+  const int in_round = min(cus_per_xcd, per_xcd - round * cus_per_xcd);
+  const int pos = round * cus_per_xcd + ((round & 1) ? in_round - 1 - j : j);
+  cells[pos * 8 + x] = (c % k_vol) * 65536 + (c / k_vol) * 8 + x;
+}
+
 __global__ void iota_kernel(int32_t *__restrict__ p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = i;
@@ -239,7 +267,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->k_vol = k_vol; p->n_in = n_in; p->n_out = n_out; p->n_pairs = n_pairs;
   p->nbr_out = p->nbr_in = nullptr; p->mask_out = p->mask_in = nullptr;
   p->perm_out = p->perm_in = nullptr;
-  p->band_count = 0; p->band_start = nullptr; p->bands_ok = false;
+  p->band_count = 0; p->band_start = nullptr; p->band_cells = nullptr; p->bands_ok = false;
   p->tile_out = p->tile_in = nullptr; p->tile_grid_out = p->tile_grid_in = 0;
   p->fwd_ok = p->dgrad_ok = false;
   p->last_stream = s;
@@ -273,6 +301,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       pool_alloc((void **)&p->mask_out, (bo ? bo : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), s) != FGMS_OK ||
+      pool_alloc((void **)&p->band_cells, (size_t)k_vol * p->band_count * sizeof(int32_t), s) != FGMS_OK ||
       pool_alloc((void **)&flags, 4 * sizeof(int), s) != FGMS_OK) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
@@ -290,6 +319,11 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   }
   band_bounds_kernel<<<(unsigned)k_vol, 128, 0, s>>>(kpos, out_map, (int)n_pairs, p->band_count,
                                                      band_rows > 0 ? band_rows : 1, p->band_start);
+  {
+    const int per_xcd = (p->band_count / 8) * k_vol;
+    band_cells_kernel<<<dim3((unsigned)((per_xcd + 255) / 256), 8), 256, 0, s>>>(
+        p->band_start, k_vol, p->band_count, num_cus() >= 8 ? num_cus() / 8 : 1, p->band_cells);
+  }
   // Reorder the rows (stable sort by offset mask), then derive the block masks
   // from the tables in their final order.  Temporaries are freed after the
   // stream synchronisation below.
@@ -411,6 +445,7 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->perm_out) pool_free(p->perm_out, p->last_stream, false);
   if (p->perm_in) pool_free(p->perm_in, p->last_stream, false);
   if (p->band_start) pool_free(p->band_start, p->last_stream, false);
+  if (p->band_cells) pool_free(p->band_cells, p->last_stream, false);
   if (p->tile_out) pool_free(p->tile_out, p->last_stream, false);
   if (p->tile_in) pool_free(p->tile_in, p->last_stream, false);
   delete p;

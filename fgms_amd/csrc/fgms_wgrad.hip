@@ -77,6 +77,7 @@ __device__ __forceinline__ half8 tr_frag(const __half *tile, int ld, int p0, int
 // pair counts, which only approximates it.  slices is a multiple of 8.
 struct SliceMap {
   const int32_t *band_start;   // [k_vol][bands + 1] or nullptr
+  const int32_t *cells;        // the plan's dispatch order of the (offset, band) cells, or nullptr
   int bands, stride;           // slice sl = bands [sl * stride, (sl + 1) * stride)
   int slices;
   int chunk;                   // > 0: plain tiles of `chunk` pairs in pair-list order instead
@@ -85,9 +86,16 @@ struct SliceMap {
 __device__ __forceinline__ bool locate_slice(const int32_t *__restrict__ kpos, const SliceMap &m,
                                              int k_vol, int block, int &k, int &first, int &count) {
   if (m.chunk > 0) return locate_tile(kpos, k_vol, m.chunk, block, k, first, count);
-  const int xcd = block % 8, idx = block / 8;
-  const int sl = (idx / k_vol) * 8 + xcd;
-  k = idx % k_vol;
+  int sl;
+  if (m.cells) {                    // biggest cells of this XCD first
+    const int cell = m.cells[block];
+    k = cell >> 16;
+    sl = cell & 0xffff;
+  } else {
+    const int xcd = block % 8, idx = block / 8;
+    sl = (idx / k_vol) * 8 + xcd;
+    k = idx % k_vol;
+  }
   if (sl >= m.slices) return false;
   const int k_first = kpos[k], k_count = kpos[k + 1] - k_first;
   if (m.band_start) {
@@ -469,6 +477,7 @@ SliceMap choose_slices(const WgradArgs &a, int ty, int stage_pairs, int64_t want
            (m.bands / (m.stride * 2)) % 8 == 0)
       m.stride *= 2;
     m.slices = (m.bands + m.stride - 1) / m.stride;
+    if (m.stride == 1) m.cells = a.plan->band_cells;
     return m;
   }
   int64_t slices = want_wgs / ((int64_t)a.k_vol * ty);
