@@ -85,10 +85,12 @@ struct Plan {
   // Only valid when every offset's pairs are ordered by output row (bands_ok).
   int band_count;
   int32_t *band_start;   // [k_vol, band_count + 1]
-  // Dispatch order of the (offset, band) cells: workgroup b of the weight gradient
-  // (XCD b % 8) takes cell band_cells[b] = offset * 65536 + band; an XCD owns the
-  // bands congruent to it mod 8 and takes its cells biggest first.
-  int32_t *band_cells;   // [k_vol * band_count]
+  // Dispatch order of the (offset, band) cells, one table per group size 1, 2, 4, 8:
+  // workgroup b of the weight gradient (XCD b % 8) takes cell
+  // band_cells[t][b] = offset * 65536 + band; an XCD owns the bands congruent to it
+  // mod 8, takes them 2^t at a time and, inside such a group, biggest cell first.
+  int32_t *band_cells;   // [4][k_vol * band_count]
+  int band_rows;         // output rows per band
   bool bands_ok;
   // Workgroup -> tile of 256 positions for the output-stationary kernel:
   // workgroup b runs on XCD b % 8 and takes tile tile_out[b] (or -1: none), chosen

@@ -190,32 +190,33 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restr
   }
 }
 
-// cells[q * 8 + xcd]: the q-th cell of XCD xcd, cell = offset * 65536 + band.  XCD x
-// owns the bands x, x + 8, ...; its cells are ranked by pair count, most first (the
-// launch ends with its longest workgroup, so those start first), ties by cell
-// number, and the ranks are laid over the CUs in a snake like the tiles above.
-// One thread per cell; a cell's rank is found by comparing with the other cells of
-// its XCD (a few hundred).
+// Dispatch order of the weight gradient's (offset, band) cells, one table per group
+// size g in {1, 2, 4, 8} (blockIdx.z): cells[q * 8 + xcd] is the q-th cell of XCD
+// xcd, cell = offset * 65536 + band.  XCD x owns the bands x, x + 8, ...; they are
+// taken g at a time (g bands x all offsets are in flight together, so g is chosen
+// at launch such that their rows fit the XCD's L2), and inside a group the cells
+// are ranked by pair count, most first (the longest workgroups start first), ties
+// by cell number.  One thread per cell; a cell's rank is found by comparing with
+// the other cells of its XCD (a few hundred).
 __global__ void band_cells_kernel(const int32_t *__restrict__ band_start, int k_vol, int bands,
-                                  int cus_per_xcd, int32_t *__restrict__ cells) {
+                                  int32_t *__restrict__ cells) {
   const int per_xcd = (bands / 8) * k_vol;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;   // cell number inside its XCD: (band / 8) * k_vol + k
-  const int x = blockIdx.y;
+  const int x = blockIdx.y, group = 1 << blockIdx.z;
   if (c >= per_xcd) return;
   auto pairs_of = [&](int cell) {
     const int k = cell % k_vol, band = (cell / k_vol) * 8 + x;
     return band_start[k * (bands + 1) + band + 1] - band_start[k * (bands + 1) + band];
   };
-  const int mine = pairs_of(c);
+  const int mine = pairs_of(c), my_group = (c / k_vol) / group;
   int rank = 0;
   for (int o = 0; o < per_xcd; ++o) {
-    const int theirs = pairs_of(o);
-    rank += (theirs > mine || (theirs == mine && o < c)) ? 1 : 0;
+    const int theirs = pairs_of(o), their_group = (o / k_vol) / group;
+    const bool before = their_group != my_group ? their_group < my_group
+                                                 : (theirs > mine || (theirs == mine && o < c));
+    rank += before ? 1 : 0;
   }
-  const int round = rank / cus_per_xcd, j = rank % cus_per_xcd;
-  const int in_round = min(cus_per_xcd, per_xcd - round * cus_per_xcd);
-  const int pos = round * cus_per_xcd + ((round & 1) ? in_round - 1 - j : j);
-  cells[pos * 8 + x] = (c % k_vol) * 65536 + (c / k_vol) * 8 + x;
+  cells[(size_t)blockIdx.z * bands * k_vol + rank * 8 + x] = (c % k_vol) * 65536 + (c / k_vol) * 8 + x;
 }
 
 __global__ void iota_kernel(int32_t *__restrict__ p, int n) {
@@ -294,6 +295,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
     p->band_count = (int)(want < 8 ? 8 : (want > kMaxBands ? kMaxBands : want));
   }
   const int band_rows = (int)((n_out + p->band_count - 1) / p->band_count);
+  p->band_rows = band_rows;
   const size_t so = (size_t)n_out * k_vol, si = (size_t)n_in * k_vol;
   const size_t bo = (size_t)(n_out + 63) / 64, bi = (size_t)(n_in + 63) / 64;
   if (pool_alloc((void **)&p->nbr_out, (so ? so : 1) * sizeof(int32_t), s) != FGMS_OK ||
@@ -301,7 +303,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       pool_alloc((void **)&p->mask_out, (bo ? bo : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), s) != FGMS_OK ||
-      pool_alloc((void **)&p->band_cells, (size_t)k_vol * p->band_count * sizeof(int32_t), s) != FGMS_OK ||
+      pool_alloc((void **)&p->band_cells, (size_t)4 * k_vol * p->band_count * sizeof(int32_t), s) != FGMS_OK ||
       pool_alloc((void **)&flags, 4 * sizeof(int), s) != FGMS_OK) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
@@ -321,8 +323,8 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
                                                      band_rows > 0 ? band_rows : 1, p->band_start);
   {
     const int per_xcd = (p->band_count / 8) * k_vol;
-    band_cells_kernel<<<dim3((unsigned)((per_xcd + 255) / 256), 8), 256, 0, s>>>(
-        p->band_start, k_vol, p->band_count, num_cus() >= 8 ? num_cus() / 8 : 1, p->band_cells);
+    band_cells_kernel<<<dim3((unsigned)((per_xcd + 255) / 256), 8, 4), 256, 0, s>>>(
+        p->band_start, k_vol, p->band_count, p->band_cells);
   }
   // Reorder the rows (stable sort by offset mask), then derive the block masks
   // from the tables in their final order.  Temporaries are freed after the

@@ -477,7 +477,13 @@ SliceMap choose_slices(const WgradArgs &a, int ty, int stage_pairs, int64_t want
            (m.bands / (m.stride * 2)) % 8 == 0)
       m.stride *= 2;
     m.slices = (m.bands + m.stride - 1) / m.stride;
-    if (m.stride == 1) m.cells = a.plan->band_cells;
+    if (m.stride == 1) {
+      // as many bands in flight per XCD as fit its 4 MB L2 (both feature matrices' rows)
+      const size_t band_bytes = (size_t)a.plan->band_rows * (a.c_in + a.c_out) * (a.dtype == FGMS_F16 ? 2 : 4);
+      int t = 3;
+      while (t > 0 && (((size_t)1 << t) * band_bytes > (size_t)7 << 19 || (1 << t) > m.bands / 8)) --t;
+      m.cells = a.plan->band_cells + (size_t)t * m.bands * a.k_vol;
+    }
     return m;
   }
   int64_t slices = want_wgs / ((int64_t)a.k_vol * ty);
