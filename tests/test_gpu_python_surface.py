@@ -120,3 +120,42 @@ def test_non_default_stream(oracle):
         be.fgms_fusion_fwd_cuda(x, w, 0, out, kpos, kpos, imap, omap, False, False)
     s.synchronize()
     G.assert_close(out.cpu().numpy(), oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"]), "fp16")
+
+
+def test_calls_can_be_captured_in_a_hip_graph(oracle):
+    """After one eager call (workspaces and the cached plan exist), forward and backward
+    record into a HIP graph: the library issues kernels only, no allocation, no memset, no
+    synchronisation.  Every replay, with eager work in between, must reproduce the eager result."""
+    import FGMS.backend as B
+    rng = np.random.default_rng(7)
+    vox = clouds.dedup(clouds._sphere_shell(rng, np.array([8., 8, 8]), 5.0, 3000), 16)
+    L = clouds.submanifold_case(vox, 64, 64, np.float16, rng)
+    D = G.to_dev(L)
+    qkpos, qsum = harness.kpos_quantized(D["knnz_host"], D["kpos"], L["k_vol"], 256)
+    out = torch.zeros(L["n_out"], 64, dtype=torch.float16, device="cuda")
+    gi = torch.zeros(L["n_in"], 64, dtype=torch.float16, device="cuda")
+    gw = torch.zeros_like(D["kernel"])
+
+    def run():
+        out.zero_(); gi.zero_(); gw.zero_()
+        B.fgms_fusion_fwd_cuda(D["in_feats"], D["kernel"], qsum, out, D["kpos"], qkpos, D["imap"], D["omap"], False, False)
+        B.fgms_bwd_cuda(D["out_grad"], D["in_feats"], D["kernel"], qsum, gi, gw, D["kpos"], qkpos,
+                        D["imap"], D["omap"], False, False)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):          # warm-up on the capture stream: plan, workspaces
+        run()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (out, gi, gw)]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run()
+    for _ in range(3):
+        out.fill_(7); gi.fill_(7); gw.fill_(7)          # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want[0]) and torch.equal(gi, want[1])
+        # the weight gradient sums its workgroups' partial tiles with fp32 atomics, whose order
+        # is not fixed: equal up to the rounding of that sum
+        G.assert_close(gw.cpu().numpy(), want[2].float().cpu().numpy(), "fp16", "replayed weight gradient")
