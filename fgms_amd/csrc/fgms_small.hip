@@ -9,9 +9,10 @@
 //     there are no atomics;
 //   * the neighbour indices of the 64 rows of a wave are one coalesced 256-byte
 //     line per offset; the gathered source rows are 8..64-byte vector loads;
-//   * all weights (k_vol * c_src * c_dst <= 13824 values) sit in LDS as fp32 and
-//     are read with wave-uniform addresses (LDS broadcast), offsets that no row
-//     of the wave uses are skipped with the plan's 64-row block mask.
+//   * the weights of an offset (c_src * c_dst <= 512 values) have one address for
+//     the whole wave and arrive through the scalar data path into scalar registers:
+//     no LDS, no barrier, one multiply-add instruction per product; offsets that no
+//     row of the wave uses are skipped with the plan's 64-row block mask.
 //
 // The reference handles these shapes with its "_once" kernels
 // (backend/spconv.cuh:569-665, 899-992), pair-stationary with scalar atomics.
@@ -22,7 +23,7 @@ namespace fgms {
 namespace {
 
 constexpr int kSmallThreads = 256;
-constexpr int kSmallMaxWeights = 13824;   // fp32 values in LDS (54 KB)
+constexpr int kSmallMaxWeights = 13824;   // values over all offsets: they stay cache-resident
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -81,51 +82,79 @@ __device__ __forceinline__ void add_store_row(T *__restrict__ p, const float (&a
   }
 }
 
-// CS / CD: source / destination channels (compile time: the inner loops unroll
-// fully and the accumulators stay in registers).
-template <typename T, int CS, int CD>
-__global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
-    const T *__restrict__ src, const T *__restrict__ w, T *__restrict__ dst,
-    const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
-    const int32_t *__restrict__ perm, int n_dst, int k_vol, bool transpose_w) {
-  extern __shared__ __align__(16) float w_lds[];   // [k_vol][CS][CD]
-  const int c_in = transpose_w ? CD : CS, c_out = transpose_w ? CS : CD;
-  for (int e = threadIdx.x; e < k_vol * CS * CD; e += kSmallThreads) {
-    const int k = e / (CS * CD), cs = (e / CD) % CS, cd = e % CD;
-    const T *wk = w + (size_t)k * c_in * c_out;
-    w_lds[e] = to_float(transpose_w ? wk[cd * c_out + cs] : wk[cs * c_out + cd]);
+// One weight of offset k as fp32, from the 32-bit words `wk` of that offset's matrix.  The
+// address is the same for every lane, so the words arrive through the scalar data path.
+template <typename T>
+__device__ __forceinline__ float weight_at(const uint32_t *__restrict__ wk, int e) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(float, wk[e]);
+  } else {
+    const uint32_t word = wk[e >> 1];
+    const unsigned short bits = (unsigned short)((e & 1) ? (word >> 16) : (word & 0xffffu));
+    return (float)__builtin_bit_cast(_Float16, bits);
   }
-  __syncthreads();
+}
+
+// CS / CD: source / destination channels (compile time: the inner loops unroll
+// fully and the accumulators stay in registers).  TR: weights are used transposed.
+template <typename T, int CS, int CD, bool TR>
+__global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
+    const T *__restrict__ src, const uint32_t *__restrict__ w, T *__restrict__ dst,
+    const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
+    const int32_t *__restrict__ perm, int n_dst) {
+  constexpr int kWordsPerOffset = CS * CD * (int)sizeof(T) / 4;
   const int row = blockIdx.x * kSmallThreads + threadIdx.x;
   const int wave_row0 = row & ~63;
   if (wave_row0 >= n_dst) return;
-  const unsigned long long mask = block_masks[wave_row0 / 64];
+  // the mask is the same for the 64 lanes: tell the compiler, so that the offset loop and
+  // the weight addresses are scalar
+  const unsigned long long mask_v = block_masks[wave_row0 / 64];
+  const unsigned long long mask =
+      ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(mask_v >> 32)) << 32) |
+      (unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)mask_v);
   if (!mask) return;
   const bool live = row < n_dst;
   float acc[CD];
 #pragma unroll
   for (int i = 0; i < CD; ++i) acc[i] = 0.f;
 
+  // Three-deep pipeline over the offsets the block uses: the neighbour index of offset
+  // t + 2 and the source row of offset t + 1 are in flight while offset t is multiplied.
+  // Every load is unconditional (lanes without a row or a pair read row 0 and drop it):
+  // the counter waits then know how many loads are outstanding and let them stay so.
   unsigned long long todo = mask;
-  int k = __builtin_ctzll(todo);
-  todo &= todo - 1;
-  int g = live ? nbr[(size_t)k * n_dst + row] : -1;
-  while (true) {
-    const int kn = todo ? __builtin_ctzll(todo) : -1;
-    if (todo) todo &= todo - 1;
-    const int gn = (kn >= 0 && live) ? nbr[(size_t)kn * n_dst + row] : -1;   // next offset's index in flight
-    if (g >= 0) {
-      float x[CS];
-      load_row<T, CS>(x, src + (size_t)g * CS);
-      const float *wk = w_lds + k * CS * CD;
+  auto next_k = [&]() {
+    if (!todo) return -1;
+    const int k = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    return k;
+  };
+  // lanes past the last row shadow it and skip the final store; an index asked for past
+  // the last offset (k < 0) is read from offset 0 and never used
+  const int row_c = live ? row : n_dst - 1;
+  auto index_of = [&](int k) { return nbr[(size_t)(k < 0 ? 0 : k) * n_dst + row_c]; };
+  auto gather = [&](float (&x)[CS], int g) { load_row<T, CS>(x, src + (size_t)(g < 0 ? 0 : g) * CS); };
+  int k0 = next_k(), k1 = next_k(), k2 = next_k();
+  int g0 = index_of(k0), g1 = index_of(k1), g2 = index_of(k2);
+  float x0[CS], x1[CS];
+  gather(x0, g0);
+  while (k0 >= 0) {
+    gather(x1, g1);                                             // next offset's row
+    const int k3 = next_k();
+    const int g3 = index_of(k3);                                // index two offsets ahead
+    const uint32_t *wk = w + (size_t)k0 * kWordsPerOffset;
+    if (g0 >= 0) {                                              // rows without a pair here sit out
 #pragma unroll
       for (int cs = 0; cs < CS; ++cs)
 #pragma unroll
-        for (int cd = 0; cd < CD; ++cd) acc[cd] += x[cs] * wk[cs * CD + cd];
+        for (int cd = 0; cd < CD; ++cd)
+          acc[cd] += x0[cs] * weight_at<T>(wk, TR ? cd * CS + cs : cs * CD + cd);
     }
-    if (kn < 0) break;
-    k = kn;
-    g = gn;
+    k0 = k1; g0 = g1;
+#pragma unroll
+    for (int i = 0; i < CS; ++i) x0[i] = x1[i];
+    k1 = k2; g1 = g2;
+    k2 = k3; g2 = g3;
   }
   // `row` is a position in the plan's row order
   if (live) add_store_row<T, CD>(dst + (size_t)(perm ? perm[row] : row) * CD, acc);
@@ -145,7 +174,8 @@ Small small_of(const GmsArgs &a) {
   s.ok = allowed(s.cs) && allowed(s.cd) && (s.cs <= 16 || s.cd <= 16) &&
          (size_t)s.cs * esz % 8 == 0 && (size_t)s.cd * esz % 8 == 0 &&
          (size_t)a.k_vol * s.cs * s.cd <= kSmallMaxWeights &&
-         reinterpret_cast<uintptr_t>(a.src) % 16 == 0 && reinterpret_cast<uintptr_t>(a.dst) % 16 == 0;
+         reinterpret_cast<uintptr_t>(a.src) % 16 == 0 && reinterpret_cast<uintptr_t>(a.dst) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(a.w) % 4 == 0;
   return s;
 }
 
@@ -156,12 +186,14 @@ int launch_small(const GmsArgs &a, const Plan *p) {
   const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
   const unsigned gx = (unsigned)((a.n_dst + kSmallThreads - 1) / kSmallThreads);
   if (gx == 0) return FGMS_OK;
-  const size_t lds = (size_t)a.k_vol * CS * CD * sizeof(float);
-  auto kern = gms_small_kernel<T, CS, CD>;
   {
     ProfileScope prof(a.transpose_w ? "gms_small_kernel(dgrad)" : "gms_small_kernel(fwd)", a.stream);
-    kern<<<gx, kSmallThreads, lds, a.stream>>>((const T *)a.src, (const T *)a.w, (T *)a.dst, nbr, masks,
-                                               perm, (int)a.n_dst, a.k_vol, a.transpose_w);
+    if (a.transpose_w)
+      gms_small_kernel<T, CS, CD, true><<<gx, kSmallThreads, 0, a.stream>>>(
+          (const T *)a.src, (const uint32_t *)a.w, (T *)a.dst, nbr, masks, perm, (int)a.n_dst);
+    else
+      gms_small_kernel<T, CS, CD, false><<<gx, kSmallThreads, 0, a.stream>>>(
+          (const T *)a.src, (const uint32_t *)a.w, (T *)a.dst, nbr, masks, perm, (int)a.n_dst);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
