@@ -16,6 +16,8 @@
 //
 // The reference handles these shapes with its "_once" kernels
 // (backend/spconv.cuh:569-665, 899-992), pair-stationary with scalar atomics.
+#include <stdlib.h>
+
 #include "fgms_device.h"
 #include "fgms_internal.h"
 
@@ -97,32 +99,46 @@ __device__ __forceinline__ float weight_at(const uint32_t *__restrict__ wk, int 
 
 // CS / CD: source / destination channels (compile time: the inner loops unroll
 // fully and the accumulators stay in registers).  TR: weights are used transposed.
+//
+// `parts` (1, 2 or 4) waves share one 64-row block: each takes every parts-th of the
+// offsets the block uses and the partial rows meet in LDS before the one update of the
+// result.  The kernel's duration is that of its longest wave (a block that uses all 27
+// offsets), and a launch of a few thousand blocks leaves the wave slots to spare.
 template <typename T, int CS, int CD, bool TR>
 __global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
     const T *__restrict__ src, const uint32_t *__restrict__ w, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
-    const int32_t *__restrict__ perm, int n_dst) {
+    const int32_t *__restrict__ perm, int n_dst, int parts) {
+  extern __shared__ __align__(16) float partial[];   // [blocks per WG][parts - 1][CD][64]
   constexpr int kWordsPerOffset = CS * CD * (int)sizeof(T) / 4;
-  const int row = blockIdx.x * kSmallThreads + threadIdx.x;
-  const int wave_row0 = row & ~63;
-  if (wave_row0 >= n_dst) return;
+  // (the wave number is the same for the 64 lanes: say so, it steers the offset loop)
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int part = wave & (parts - 1), block_in_wg = wave / parts;
+  const int block = blockIdx.x * (kSmallThreads / 64 / parts) + block_in_wg;
+  const int row = block * 64 + lane;
+  const bool live = row < n_dst;
   // the mask is the same for the 64 lanes: tell the compiler, so that the offset loop and
   // the weight addresses are scalar
-  const unsigned long long mask_v = block_masks[wave_row0 / 64];
+  const unsigned long long mask_v = (size_t)block * 64 < (size_t)n_dst ? block_masks[block] : 0ull;
   const unsigned long long mask =
       ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(mask_v >> 32)) << 32) |
       (unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)mask_v);
-  if (!mask) return;
-  const bool live = row < n_dst;
+  // this wave's share: the set bits number part, part + parts, ...
+  unsigned long long todo = mask;
+  if (parts > 1) {
+    todo = 0;
+    int i = 0;
+    for (unsigned long long m = mask; m; m &= m - 1, ++i)
+      if ((i & (parts - 1)) == part) todo |= m & (0 - m);
+  }
   float acc[CD];
 #pragma unroll
   for (int i = 0; i < CD; ++i) acc[i] = 0.f;
 
-  // Three-deep pipeline over the offsets the block uses: the neighbour index of offset
-  // t + 2 and the source row of offset t + 1 are in flight while offset t is multiplied.
-  // Every load is unconditional (lanes without a row or a pair read row 0 and drop it):
-  // the counter waits then know how many loads are outstanding and let them stay so.
-  unsigned long long todo = mask;
+  // Three-deep pipeline over the offsets: the neighbour index of offset t + 2 and the
+  // source row of offset t + 1 are in flight while offset t is multiplied.  Every load is
+  // unconditional (lanes without a row or a pair read row 0 and drop it): the counter
+  // waits then know how many loads are outstanding and let them stay so.
   auto next_k = [&]() {
     if (!todo) return -1;
     const int k = __builtin_ctzll(todo);
@@ -134,30 +150,47 @@ __global__ __launch_bounds__(kSmallThreads) void gms_small_kernel(
   const int row_c = live ? row : n_dst - 1;
   auto index_of = [&](int k) { return nbr[(size_t)(k < 0 ? 0 : k) * n_dst + row_c]; };
   auto gather = [&](float (&x)[CS], int g) { load_row<T, CS>(x, src + (size_t)(g < 0 ? 0 : g) * CS); };
-  int k0 = next_k(), k1 = next_k(), k2 = next_k();
-  int g0 = index_of(k0), g1 = index_of(k1), g2 = index_of(k2);
-  float x0[CS], x1[CS];
-  gather(x0, g0);
-  while (k0 >= 0) {
-    gather(x1, g1);                                             // next offset's row
-    const int k3 = next_k();
-    const int g3 = index_of(k3);                                // index two offsets ahead
-    const uint32_t *wk = w + (size_t)k0 * kWordsPerOffset;
-    if (g0 >= 0) {                                              // rows without a pair here sit out
+  int k0 = next_k();
+  if (k0 >= 0) {
+    int k1 = next_k(), k2 = next_k();
+    int g0 = index_of(k0), g1 = index_of(k1), g2 = index_of(k2);
+    float x0[CS], x1[CS];
+    gather(x0, g0);
+    while (k0 >= 0) {
+      gather(x1, g1);                                             // next offset's row
+      const int k3 = next_k();
+      const int g3 = index_of(k3);                                // index two offsets ahead
+      const uint32_t *wk = w + (size_t)k0 * kWordsPerOffset;
+      if (g0 >= 0) {                                              // rows without a pair here sit out
 #pragma unroll
-      for (int cs = 0; cs < CS; ++cs)
+        for (int cs = 0; cs < CS; ++cs)
 #pragma unroll
-        for (int cd = 0; cd < CD; ++cd)
-          acc[cd] += x0[cs] * weight_at<T>(wk, TR ? cd * CS + cs : cs * CD + cd);
+          for (int cd = 0; cd < CD; ++cd)
+            acc[cd] += x0[cs] * weight_at<T>(wk, TR ? cd * CS + cs : cs * CD + cd);
+      }
+      k0 = k1; g0 = g1;
+#pragma unroll
+      for (int i = 0; i < CS; ++i) x0[i] = x1[i];
+      k1 = k2; g1 = g2;
+      k2 = k3; g2 = g3;
     }
-    k0 = k1; g0 = g1;
-#pragma unroll
-    for (int i = 0; i < CS; ++i) x0[i] = x1[i];
-    k1 = k2; g1 = g2;
-    k2 = k3; g2 = g3;
   }
-  // `row` is a position in the plan's row order
-  if (live) add_store_row<T, CD>(dst + (size_t)(perm ? perm[row] : row) * CD, acc);
+  if (parts > 1) {
+    float *mine = partial + ((size_t)(block_in_wg * (parts - 1) + part - 1) * CD) * 64 + lane;
+    if (part != 0) {
+#pragma unroll
+      for (int cd = 0; cd < CD; ++cd) mine[cd * 64] = acc[cd];
+    }
+    __syncthreads();
+    if (part != 0) return;
+    for (int p = 0; p < parts - 1; ++p) {
+      const float *theirs = partial + ((size_t)(block_in_wg * (parts - 1) + p) * CD) * 64 + lane;
+#pragma unroll
+      for (int cd = 0; cd < CD; ++cd) acc[cd] += theirs[cd * 64];
+    }
+  }
+  // `row` is a position in the plan's row order; a block no pair touches leaves its rows alone
+  if (live && mask) add_store_row<T, CD>(dst + (size_t)(perm ? perm[row] : row) * CD, acc);
 }
 
 struct Small {
@@ -184,16 +217,28 @@ int launch_small(const GmsArgs &a, const Plan *p) {
   const int32_t *nbr = a.transpose_w ? p->nbr_in : p->nbr_out;
   const unsigned long long *masks = a.transpose_w ? p->mask_in : p->mask_out;
   const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
-  const unsigned gx = (unsigned)((a.n_dst + kSmallThreads - 1) / kSmallThreads);
-  if (gx == 0) return FGMS_OK;
+  if (a.n_dst == 0) return FGMS_OK;
+  // waves per 64-row block: four while the launch is a couple of rounds of the chip's wave
+  // slots (200k rows: 23 us against 27 us with one wave per block), one when the rounds
+  // are many and the longest wave no longer decides
+  const size_t blocks = ((size_t)a.n_dst + 63) / 64;
+  const size_t slots = (size_t)num_cus() * 4 * 7;
+  int parts = blocks <= slots ? 4 : blocks <= 2 * slots ? 2 : 1;
+  if (const char *e = getenv("FGMS_SMALL_PARTS")) {   // 1, 2 or 4: overrides the choice
+    const int v = atoi(e);
+    if (v == 1 || v == 2 || v == 4) parts = v;
+  }
+  const int blocks_per_wg = kSmallThreads / 64 / parts;
+  const unsigned gx = (unsigned)((blocks + blocks_per_wg - 1) / blocks_per_wg);
+  const size_t lds = parts > 1 ? (size_t)blocks_per_wg * (parts - 1) * CD * 64 * sizeof(float) : 0;
   {
     ProfileScope prof(a.transpose_w ? "gms_small_kernel(dgrad)" : "gms_small_kernel(fwd)", a.stream);
     if (a.transpose_w)
-      gms_small_kernel<T, CS, CD, true><<<gx, kSmallThreads, 0, a.stream>>>(
-          (const T *)a.src, (const uint32_t *)a.w, (T *)a.dst, nbr, masks, perm, (int)a.n_dst);
+      gms_small_kernel<T, CS, CD, true><<<gx, kSmallThreads, lds, a.stream>>>(
+          (const T *)a.src, (const uint32_t *)a.w, (T *)a.dst, nbr, masks, perm, (int)a.n_dst, parts);
     else
-      gms_small_kernel<T, CS, CD, false><<<gx, kSmallThreads, 0, a.stream>>>(
-          (const T *)a.src, (const uint32_t *)a.w, (T *)a.dst, nbr, masks, perm, (int)a.n_dst);
+      gms_small_kernel<T, CS, CD, false><<<gx, kSmallThreads, lds, a.stream>>>(
+          (const T *)a.src, (const uint32_t *)a.w, (T *)a.dst, nbr, masks, perm, (int)a.n_dst, parts);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;

@@ -91,6 +91,16 @@ def test_submanifold_wide_wave_tiles(capi, oracle, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("parts", [1, 2, 4])
+@pytest.mark.parametrize("shape", [(4, 32), (16, 16), (64, 8)], ids=lambda s: "%dx%d" % s)
+def test_skinny_layers_by_waves_per_block(capi, oracle, monkeypatch, shape, parts, dtype):
+    """The skinny-channel kernel with one, two and four waves sharing a 64-row block (the
+    library picks by the size of the launch; FGMS_SMALL_PARTS, read on every call, overrides)."""
+    monkeypatch.setenv("FGMS_SMALL_PARTS", str(parts))
+    check_all(capi, oracle, layer(17, *shape, dtype), policy=0, use_plan=True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
 @pytest.mark.parametrize("kind,shape", [("down", (64, 128)), ("up", (128, 64)), ("down", (16, 32)), ("up", (5, 3))])
 def test_strided_and_transposed(capi, oracle, kind, shape, dtype):
     L = layer(14, shape[0], shape[1], dtype, kind)
