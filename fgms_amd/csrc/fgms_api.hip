@@ -246,13 +246,32 @@ int check_common(const void *a, const void *b, const void *c, const int32_t *kpo
   return FGMS_OK;
 }
 
+// The output-stationary kernel multiplies every (64-row block, offset) combination in
+// use, 64 row slots each, whether or not a row has a pair there; the pair-stationary one
+// multiplies pairs only and pays with an atomic per result element.  Measured on MI355X
+// the atomics cost about as much as 240 (fp16) / 64 (fp32) channels of contraction per
+// pair, so the pair-stationary kernel wins when
+//   c_src + that  <  c_src * slots / pairs        (with 15 % in favour of the kernel
+// without atomics, whose results do not depend on the run).  Of the usual layers only wide
+// ones over scattered clouds qualify (256 -> 256 over a 50 k subsample: slots / pairs 2.6).
+bool sparse_rows(const GmsArgs &a, const Plan *plan) {
+  const int stages = a.transpose_w ? plan->stages_in : plan->stages_out;
+  if (stages <= 0 || a.n_pairs <= 0) return false;
+  const double slots_per_pair = (double)stages * 64.0 / (double)a.n_pairs;
+  const double c_src = a.transpose_w ? a.c_out : a.c_in;
+  const double atomics = a.dtype == FGMS_F16 ? 240.0 : 64.0;
+  return (c_src + atomics) * 1.15 < c_src * slots_per_pair;
+}
+
 int run_gms(GmsArgs a, const Plan *plan) {
   if (plan) plan->last_stream = a.stream;
   const bool dense = a.dense_k >= 0;
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
   if (g_policy != 1) {
-    if (!dense && g_policy == 0 && small_gms_supported(a, plan)) return launch_small_gms(a, plan);
-    if (!dense && g_policy != 2 && planned_gms_supported(a, plan)) return launch_planned_gms(a, plan);
+    if (!dense && (g_policy == 0 || g_policy == 4) && small_gms_supported(a, plan)) return launch_small_gms(a, plan);
+    if (!dense && g_policy != 2 && planned_gms_supported(a, plan) &&
+        !(g_policy != 4 && sparse_rows(a, plan) && mfma_gms_supported(a)))
+      return launch_planned_gms(a, plan);
     if (mfma_gms_supported(a)) return launch_mfma_gms(a);
   }
   return launch_generic_gms(a);

@@ -99,6 +99,9 @@ struct Plan {
   int32_t *tile_out, *tile_in;
   int tile_grid_out, tile_grid_in;   // entries of the tables (a multiple of 8)
   mutable hipStream_t last_stream;   // the stream of the latest launch that read the plan
+  // (64-row block, offset) combinations with at least one pair: the output-stationary
+  // kernels run stages * 64 row slots for n_pairs pairs
+  int stages_out, stages_in;
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };

@@ -132,7 +132,12 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
  * 1 = force the generic (non-MFMA) kernels, 2 = force the pair-stationary MFMA
  * kernels even when a usable plan is passed, 3 = automatic dispatch but the
  * output-stationary kernel uses its 128-column wave tiles whenever the layer
- * has a multiple of 128 output channels (normally only large fp16 layers).
+ * has a multiple of 128 output channels (normally only large fp16 layers),
+ * 4 = automatic dispatch but never the pair-stationary kernel where the
+ * output-stationary one can run: forward and input-gradient results are then the
+ * same bit for bit from run to run (automatic dispatch gives wide layers over
+ * scattered clouds, with few pairs per 64-row block and offset, to the
+ * pair-stationary kernel, whose atomic sums depend on their order).
  * Process-wide. */
 void fgms_set_kernel_policy(int policy);
 

@@ -227,6 +227,41 @@ def test_baseline_configs_scaled(capi, oracle, cfg, variant):
     check_all(capi, oracle, L, policy=0, use_plan=False)
 
 
+@pytest.mark.parametrize("dtype", ["wide", "wide-fp32"], ids=["fp16", "fp32"])
+def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dtype):
+    """A 256 -> 256 layer over a scattered cloud (few pairs per 64-row block and offset):
+    automatic dispatch weighs the empty row slots of the output-stationary kernel against
+    the atomics of the pair-stationary one and picks the latter; a dense 64 -> 64 layer
+    stays output-stationary.  Results against the oracle either way."""
+    L = clouds.config_case(5, dtype, scale=0.08)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(0)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    capi.profile_reset()
+    capi.profile_enable(True)
+    out = G.run_fwd(capi, D, fused=True, plan=plan)
+    torch.cuda.synchronize()
+    capi.profile_enable(False)
+    names = [n for n, _ in capi.profile_records()]
+    capi.profile_reset()
+    plan.close()
+    assert "gms_pairs_kernel(fwd)" in names and "gms_rows_kernel(fwd)" not in names, names
+    ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
+    G.assert_close(out, ref, G.mode_of(L["in_feats"].dtype, False), "fwd")
+
+    L = layer(5, 64, 64, np.float16)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    capi.profile_enable(True)
+    G.run_fwd(capi, D, fused=True, plan=plan)
+    torch.cuda.synchronize()
+    capi.profile_enable(False)
+    names = [n for n, _ in capi.profile_records()]
+    capi.profile_reset()
+    plan.close()
+    assert "gms_rows_kernel(fwd)" in names, names
+
+
 def test_config2_scaled_fp32_and_tf32(capi, oracle):
     L = clouds.config_case(2, scale=0.08)
     check_all(capi, oracle, L, policy=0, use_plan=True, arch80=False)
