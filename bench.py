@@ -162,10 +162,15 @@ def main():
         if "fwd" in passes:
             capi.fusion_fwd(D["in_feats"], D["kernel"], 0, out, D["kpos"], None, D["imap"], D["omap"],
                             False, arch80, plan=plan)
-        if "dgrad" in passes:
-            capi.dgrad(D["out_grad"], D["kernel"], gi, D["kpos"], D["imap"], D["omap"], plan=plan)
-        if "wgrad" in passes:
-            capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
+        if "dgrad" in passes and "wgrad" in passes:
+            # both gradients in one call, as the reference's fgms_bwd_cuda computes them
+            capi.bwd(D["out_grad"], D["in_feats"], D["kernel"], 0, gi, gw, D["kpos"], None,
+                     D["imap"], D["omap"], False, arch80, plan=plan)
+        else:
+            if "dgrad" in passes:
+                capi.dgrad(D["out_grad"], D["kernel"], gi, D["kpos"], D["imap"], D["omap"], plan=plan)
+            if "wgrad" in passes:
+                capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
 
     if args.copy_calib:
         a_ = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")

@@ -263,18 +263,29 @@ bool sparse_rows(const GmsArgs &a, const Plan *plan) {
   return (c_src + atomics) * 1.15 < c_src * slots_per_pair;
 }
 
+enum class Route { kSkinny, kRows, kPairs, kGeneric };
+
+// Which kernel a forward / input-gradient pass takes.
+Route route_of(const GmsArgs &a, const Plan *plan) {
+  const bool dense = a.dense_k >= 0;
+  if (g_policy == 1) return Route::kGeneric;
+  if (!dense && (g_policy == 0 || g_policy == 4) && small_gms_supported(a, plan)) return Route::kSkinny;
+  if (!dense && g_policy != 2 && planned_gms_supported(a, plan) &&
+      !(g_policy != 4 && sparse_rows(a, plan) && mfma_gms_supported(a)))
+    return Route::kRows;
+  return mfma_gms_supported(a) ? Route::kPairs : Route::kGeneric;
+}
+
 int run_gms(GmsArgs a, const Plan *plan) {
   if (plan) plan->last_stream = a.stream;
   const bool dense = a.dense_k >= 0;
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
-  if (g_policy != 1) {
-    if (!dense && (g_policy == 0 || g_policy == 4) && small_gms_supported(a, plan)) return launch_small_gms(a, plan);
-    if (!dense && g_policy != 2 && planned_gms_supported(a, plan) &&
-        !(g_policy != 4 && sparse_rows(a, plan) && mfma_gms_supported(a)))
-      return launch_planned_gms(a, plan);
-    if (mfma_gms_supported(a)) return launch_mfma_gms(a);
+  switch (route_of(a, plan)) {
+    case Route::kSkinny: return launch_small_gms(a, plan);
+    case Route::kRows: return launch_planned_gms(a, plan);
+    case Route::kPairs: return launch_mfma_gms(a);
+    default: return launch_generic_gms(a);
   }
-  return launch_generic_gms(a);
 }
 
 int run_wgrad(const WgradArgs &a) {
@@ -447,11 +458,47 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
              int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs,
              int dtype, fgms_plan_t *plan, void *stream) {
   (void)sum_nnz; (void)qkpos; (void)separate_mid; (void)arch80;
-  int rc = fgms_dgrad(out_feats_grad, kernel, in_feats_grad, kpos, in_map, out_map, n_in, n_out,
-                      c_in, c_out, k_vol, n_pairs, dtype, plan, stream);
+  int rc = check_common(out_feats_grad, kernel, in_feats_grad, kpos, in_map, out_map, n_in, n_out,
+                        c_in, c_out, k_vol, n_pairs, dtype);
   if (rc) return rc;
-  return fgms_wgrad(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
-                    c_in, c_out, k_vol, n_pairs, dtype, plan, stream);
+  if ((rc = check_common(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
+                         c_in, c_out, k_vol, n_pairs, dtype)))
+    return rc;
+  const Plan *p = (const Plan *)plan;
+  GmsArgs d{};
+  d.src = out_feats_grad; d.w = kernel; d.dst = in_feats_grad; d.kpos = kpos;
+  d.gmap = out_map; d.smap = in_map;   // roles swap, as at backend/spconv.cu:460,559
+  d.n_src = n_out; d.n_dst = n_in; d.c_in = c_in; d.c_out = c_out; d.k_vol = k_vol;
+  d.n_pairs = n_pairs; d.transpose_w = true; d.dense_k = -1; d.n_dense = 0; d.dtype = dtype;
+  d.stream = (hipStream_t)stream;
+  WgradArgs w{};
+  w.in = in_feats; w.gout = out_feats_grad; w.gw = kernel_grad; w.kpos = kpos;
+  w.imap = in_map; w.omap = out_map; w.n_in = n_in; w.n_out = n_out; w.c_in = c_in;
+  w.c_out = c_out; w.k_vol = k_vol; w.n_pairs = n_pairs; w.dtype = dtype;
+  w.stream = (hipStream_t)stream;
+  w.plan = p;
+  // Both gradients through their main kernels: two launches instead of four.  The weight
+  // gradient goes first and its launch also re-lays the weights for the input gradient,
+  // whose launch in turn also rounds the weight gradient's fp32 sums into the caller's
+  // fp16 tensor.  (The two gradients do not depend on each other.)
+  if (n_pairs > 0 && route_of(d, p) == Route::kRows && g_policy != 1 && mfma_wgrad_supported(w)) {
+    p->last_stream = d.stream;
+    SideJob pack{}, flush{};
+    const void *packed = nullptr;
+    if ((rc = planned_pack_job(d, &pack, &packed))) return rc;
+    w.side = pack;
+    w.deferred_flush = &flush;
+    if ((rc = launch_mfma_wgrad(w))) return rc;
+    d.prepacked = packed;
+    d.side = flush;
+    if ((rc = launch_planned_gms(d, p))) {
+      (void)launch_side_job(flush, d.stream);   // the accumulator must not stay filled
+      return rc;
+    }
+    return FGMS_OK;
+  }
+  if ((rc = run_gms(d, p))) return rc;
+  return run_wgrad(w);
 }
 
 int fgms_build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords,

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fgms_internal.h"
+
 namespace fgms {
 
 // Offset k is cut into ceil(n_k / rows) tiles; tiles are numbered offset by
@@ -59,6 +61,63 @@ __device__ __forceinline__ void atomic_add(__half *addr, float v) {
 // Packed fp16x2 accumulate (global_atomic_pk_add_f16); addr must be 4-byte aligned.
 __device__ __forceinline__ void atomic_add_pk(__half *addr, float lo, float hi) {
   unsafeAtomicAdd(reinterpret_cast<__half2 *>(addr), __floats2half2_rn(lo, hi));
+}
+
+// Weight re-layout into per-lane MFMA fragment order.  packed[k][q][nt][lane][e],
+// q = slab * S + s, E = elements per 16-byte chunk:
+//   source channel  cs = slab * 2*S*E + (lane / 32) * S*E + s * E + e
+//   dest   channel  cd = nt * 32 + lane % 32
+//   value = transpose ? W[k][cd][cs] : W[k][cs][cd]
+// Elements first, first + stride, ... of the packed array.
+template <typename T>
+__device__ __forceinline__ void pack_weight_elements(const T *__restrict__ w, T *__restrict__ packed,
+                                                     int k_vol, int c_in, int c_out, int S,
+                                                     bool transpose, size_t first, size_t stride) {
+  constexpr int E = 16 / (int)sizeof(T);
+  const int c_src = transpose ? c_out : c_in;
+  const int c_dst = transpose ? c_in : c_out;
+  const size_t per_k = (size_t)c_src * c_dst;
+  const size_t total = per_k * k_vol;
+  const int nts = c_dst / 32;
+  for (size_t i = first; i < total; i += stride) {
+    const int k = (int)(i / per_k);
+    size_t r = i % per_k;
+    const int e = (int)(r % E); r /= E;
+    const int lane = (int)(r % 64); r /= 64;
+    const int nt = (int)(r % nts); r /= nts;
+    const int q = (int)r;
+    const int slab = q / S, s = q % S;
+    const int cs = slab * 2 * S * E + (lane / 32) * S * E + s * E + e;
+    const int cd = nt * 32 + lane % 32;
+    const T *wk = w + (size_t)k * c_in * c_out;
+    packed[i] = transpose ? wk[(size_t)cd * c_out + cs] : wk[(size_t)cs * c_out + cd];
+  }
+}
+
+// dst[i] += acc[i] rounded once to fp16, and acc[i] is reset: the accumulator is handed
+// back all-zero, which is the state the next weight gradient expects to find it in.
+__device__ __forceinline__ void add_and_clear_elements(__half *__restrict__ dst, float *__restrict__ acc,
+                                                       size_t n, size_t first, size_t stride) {
+  for (size_t i = first; i < n; i += stride) {
+    dst[i] = __float2half(__half2float(dst[i]) + acc[i]);
+    acc[i] = 0.f;
+  }
+}
+
+// The side job of a launch, run by workgroup `block` of its job.blocks workgroups.
+__device__ __forceinline__ void run_side_job(const SideJob &job, int block) {
+  const size_t first = (size_t)block * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)job.blocks * blockDim.x;
+  if (job.kind == 1) {
+    if (job.dtype == FGMS_F16)
+      pack_weight_elements<__half>((const __half *)job.src, (__half *)job.dst, job.k_vol, job.c_in,
+                                   job.c_out, job.S, job.transpose != 0, first, stride);
+    else
+      pack_weight_elements<float>((const float *)job.src, (float *)job.dst, job.k_vol, job.c_in,
+                                  job.c_out, job.S, job.transpose != 0, first, stride);
+  } else if (job.kind == 2) {
+    add_and_clear_elements((__half *)job.dst, job.acc, job.n, first, stride);
+  }
 }
 
 }  // namespace fgms

@@ -27,6 +27,23 @@ void set_error(const char *fmt, ...);
 //          op(W) = W            (c_src = c_in,  c_dst = c_out)
 // dgrad:   src = out_grad, dst = in_grad, gmap = out_map, smap = in_map,
 //          op(W) = W^T          (c_src = c_out, c_dst = c_in)
+// A small job that rides along with a big launch instead of costing a launch of its own:
+// the first `blocks` workgroups (x) of the grid run it and exit, the rest see their index
+// lowered by `blocks`.  A multiple of 8, so that a workgroup keeps its XCD (index mod 8).
+//   kind 1: re-lay the weights `src` into MFMA fragment order at `dst` (what
+//           pack_weights_kernel does), for the launch that follows on the stream;
+//   kind 2: dst[i] += acc[i] rounded once to fp16 and acc[i] = 0 (what add_and_clear_kernel
+//           does) for the fp32 accumulator the previous launch on the stream filled.
+struct SideJob {
+  int kind;      // 0: none
+  int blocks;
+  const void *src;
+  void *dst;
+  float *acc;
+  size_t n;      // elements
+  int k_vol, c_in, c_out, S, transpose, dtype;
+};
+
 // dense:   gmap == smap == nullptr means the identity map over n_dense rows of
 //          the single offset `dense_k` (the separately handled centre offset).
 struct GmsArgs {
@@ -45,6 +62,8 @@ struct GmsArgs {
   int64_t n_dense;
   int dtype;
   hipStream_t stream;
+  const void *prepacked;   // output-stationary kernel only: the weights are already re-laid here
+  SideJob side;            // ... and this rides along with its launch
 };
 
 struct WgradArgs {
@@ -60,6 +79,10 @@ struct WgradArgs {
   int dtype;
   hipStream_t stream;
   const struct Plan *plan;   // optional
+  SideJob side;              // MFMA kernels only: rides along with the launch
+  // MFMA kernels, fp16: do not launch the fp32 -> fp16 flush of the accumulator; describe
+  // it in *deferred_flush instead, for the caller to attach to its next launch
+  SideJob *deferred_flush;
 };
 
 // Plan: neighbour tables built from the pair lists.
@@ -137,6 +160,11 @@ int num_cus();         // compute units of the current device
 int launch_mfma_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);
+// Describes the weight re-layout the output-stationary kernel needs for `a` as a side job
+// (nothing is launched) and returns where the packed weights will be.
+int planned_pack_job(const GmsArgs &a, SideJob *job, const void **packed);
+// Runs a side job in a launch of its own.
+int launch_side_job(const SideJob &job, hipStream_t stream);
 bool small_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_small_gms(const GmsArgs &a, const Plan *p);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);

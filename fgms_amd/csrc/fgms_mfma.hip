@@ -25,6 +25,8 @@
 // Gathered rows reach LDS with 16-byte loads, 2*S lanes per row (full 128-byte
 // lines for S = 4), in an XOR-swizzled layout so that the b128 reads of the MFMA
 // operand do not collide on banks.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "fgms_device.h"
@@ -56,34 +58,16 @@ __device__ __forceinline__ int a_slot(int row, int c) {
 }
 
 // ---------------------------------------------------------------------------
-// Weight re-layout.  packed[k][q][nt][lane][e], q = slab * S + s:
-//   source channel  cs = slab * 2*S*E + (lane / 32) * S*E + s * E + e
-//   dest   channel  cd = nt * 32 + lane % 32
-//   value = transpose ? W[k][cd][cs] : W[k][cs][cd]
+// Weight re-layout (see pack_weight_elements) in a launch of its own.
 template <typename T>
 __global__ void pack_weights_kernel(const T *__restrict__ w, T *__restrict__ packed, int k_vol,
                                     int c_in, int c_out, int S, bool transpose) {
-  constexpr int E = Elem<T>::per_chunk;
-  const int c_src = transpose ? c_out : c_in;
-  const int c_dst = transpose ? c_in : c_out;
-  const size_t per_k = (size_t)c_src * c_dst;
-  const size_t total = per_k * k_vol;
-  const int nts = c_dst / 32;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (size_t)gridDim.x * blockDim.x) {
-    const int k = (int)(i / per_k);
-    size_t r = i % per_k;
-    const int e = (int)(r % E); r /= E;
-    const int lane = (int)(r % 64); r /= 64;
-    const int nt = (int)(r % nts); r /= nts;
-    const int q = (int)r;
-    const int slab = q / S, s = q % S;
-    const int cs = slab * 2 * S * E + (lane / 32) * S * E + s * E + e;
-    const int cd = nt * 32 + lane % 32;
-    const T *wk = w + (size_t)k * c_in * c_out;
-    packed[i] = transpose ? wk[(size_t)cd * c_out + cs] : wk[(size_t)cs * c_out + cd];
-  }
+  pack_weight_elements<T>(w, packed, k_vol, c_in, c_out, S, transpose,
+                          (size_t)blockIdx.x * blockDim.x + threadIdx.x,
+                          (size_t)gridDim.x * blockDim.x);
 }
+
+__global__ void side_job_kernel(SideJob job) { run_side_job(job, blockIdx.x); }
 
 // Copies the packed weights of offset k, destination tiles [nt0, nt0 + NT), to LDS.
 template <int NT>
@@ -136,6 +120,57 @@ __device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__
     int4v b[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[((slab * S + s) * NT + nt) * 64 + lane];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+    }
+  }
+}
+
+// --- forward weights straight from the caller's tensor (fp16) -----------------------
+// The forward pass contracts over the ROWS of W[k] (W[k][cs][cd], cd contiguous) while an
+// MFMA lane wants 8 consecutive cs of one cd.  Instead of re-laying the weights in a launch
+// of their own, a stage's weight tile (2*S*8 rows cs x NT*32 columns cd) goes to LDS as it
+// lies in memory, in 16-byte chunks, and the fragments come out through the transposing
+// LDS read.  Chunk c of row `row` sits at chunk position c ^ raw_swizzle(row): the four
+// consecutive rows one transposing read touches then cover all banks once.
+template <int NT>
+__device__ __forceinline__ int raw_swizzle(int row) {
+  if constexpr (NT == 4) return (row & 3) << 2;          // 256-byte rows
+  else if constexpr (NT == 2) return ((row >> 1) & 1) << 2;   // 128-byte rows
+  else return 0;                                          // 64-byte rows
+}
+
+// B fragment of MFMA step s, 32-column tile nt: the 8 values W[(h*S + s)*8 + 0..7][nt*32 + lane%32].
+template <int NT, int S>
+__device__ __forceinline__ int4v raw_weight_frag(const int4v *__restrict__ w_lds, int s, int nt, int lane) {
+  constexpr int RS = NT * 4;                              // chunks per row
+  const int b = lane >> 4, i = lane & 15, h = lane >> 5;
+  const int row = (h * S + s) * 8 + (i >> 2);
+  const int chunk = nt * 4 + (b & 1) * 2 + ((i & 3) >> 1);
+  const __half *base = reinterpret_cast<const __half *>(w_lds) +
+                       ((size_t)row * RS + (chunk ^ raw_swizzle<NT>(row))) * 8 + (i & 1) * 4;
+  typedef short short4v __attribute__((ext_vector_type(4)));
+  typedef short short8v __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) short4v lds_v4;
+  const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4 *)(base));
+  const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4 *)(base + 4 * RS * 8));   // rows + 4: same swizzle
+  const short8v v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(int4v, v);
+}
+
+// acc[mt][nt] += A(slab) x W(slab), weights as raw_weight_frag reads them.
+template <typename T, int NT, int S>
+__device__ __forceinline__ void mma_slab_raw(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+                                             const int4v *__restrict__ w_lds, int lane) {
+  const int h = lane / 32, r = lane % 32;
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    int4v b[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) b[nt] = raw_weight_frag<NT, S>(w_lds, s, nt, lane);
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
       const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
@@ -446,12 +481,23 @@ __device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (
   }
 }
 
-template <typename T, int NT, int S>
+// RAW: `packed` is the caller's weight tensor itself (forward, fp16: see raw_weight_frag);
+// otherwise the re-laid copy pack_weight_elements makes.
+template <typename T, int NT, int S, bool RAW>
 __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
-    int c_src, int c_dst, int part_stages) {
+    int c_src, int c_dst, int part_stages, SideJob side) {
+  // the leading workgroups of the grid run the side job, if there is one
+  int block_x = blockIdx.x;
+  if (side.blocks) {
+    if (block_x < side.blocks) {
+      if (blockIdx.y == 0 && blockIdx.z == 0) run_side_job(side, block_x);
+      return;
+    }
+    block_x -= side.blocks;
+  }
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
   constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
@@ -470,7 +516,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   const int4v *packed4 = reinterpret_cast<const int4v *>(packed);
   const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
 
-  const int tile = tile_order ? tile_order[blockIdx.x] : (int)blockIdx.x;
+  const int tile = tile_order ? tile_order[block_x] : block_x;
   if (tile < 0) return;
   const int row0 = tile * kTileRows + wave * kWaveRows;
   const int my_row = row0 + lane;
@@ -529,8 +575,16 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     for (int i = 0; i < NW; ++i) {
       const int e = threadIdx.x + kThreads * i;
       if (NW * kThreads == WCH || e < WCH) {
-        const int q = e / (NT * 64), rem = e % (NT * 64);
-        wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
+        if constexpr (RAW) {
+          // chunk e of the tile as it lies in memory: row e / (NT*4) of the slab's 2*S*8
+          // rows of W[k], 16-byte piece e % (NT*4) of the NT*32 columns from nt0*32 on
+          const int row = e / (NT * 4), c = e % (NT * 4);
+          wreg[i] = *reinterpret_cast<const int4v *>(
+              packed + ((size_t)k * c_src + slab * (C * E) + row) * c_dst + nt0 * 32 + c * E);
+        } else {
+          const int q = e / (NT * 64), rem = e % (NT * 64);
+          wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
+        }
       }
     }
   };
@@ -538,7 +592,14 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
 #pragma unroll
     for (int i = 0; i < NW; ++i) {
       const int e = threadIdx.x + kThreads * i;
-      if (NW * kThreads == WCH || e < WCH) w_lds[buf * WCH + e] = wreg[i];
+      if (NW * kThreads == WCH || e < WCH) {
+        if constexpr (RAW) {
+          const int row = e / (NT * 4), c = e % (NT * 4);
+          w_lds[buf * WCH + row * (NT * 4) + (c ^ raw_swizzle<NT>(row))] = wreg[i];
+        } else {
+          w_lds[buf * WCH + e] = wreg[i];
+        }
+      }
     }
   };
 
@@ -576,7 +637,10 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
       weights_issue(wreg, nk, nslab);
       if (next_active) gather_issue<T, S>(v, gsel, gidx, src, c_src, nslab, lane);
     }
-    if (active) mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+    if (active) {
+      if constexpr (RAW) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+      else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+    }
     if (!has_next) break;
     wave_lds_fence();
     if (next_active) gather_commit<S>(a_lds, v, gsel, lane);
@@ -678,16 +742,31 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   return FGMS_OK;
 }
 
+// FGMS_RAW_WEIGHTS=0 keeps the forward pass on re-laid weights (for comparison).
+bool raw_weights_enabled() {
+  static const bool on = !(getenv("FGMS_RAW_WEIGHTS") && atoi(getenv("FGMS_RAW_WEIGHTS")) == 0);
+  return on;
+}
+
 template <typename T, int NT, int S>
 int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
                 const unsigned long long *masks, const int32_t *perm, const int32_t *tile_order,
                 int tile_grid) {
-  const T *packed = nullptr;
-  int rc = pack_weights<T>(a, s, &packed);
-  if (rc != FGMS_OK) return rc;
+  // fp16 forward reads the weight tensor as it is (16-byte aligned rows of the tile);
+  // everything else gets a re-laid copy, made here unless the caller already has one.
+  // (With 128-column wave tiles the transposing reads cost more than the re-layout
+  // launch they save: 128 -> 128 over 120k voxels, 99.7 us against 93.6 + 4.4 us.)
+  constexpr bool kCanRaw = sizeof(T) == 2 && NT != 4;
+  const bool raw = kCanRaw && !a.transpose_w && !a.prepacked &&
+                   reinterpret_cast<uintptr_t>(a.w) % 16 == 0 && raw_weights_enabled();
+  const T *packed = raw ? (const T *)a.w : (const T *)a.prepacked;
+  if (!packed) {
+    int rc = pack_weights<T>(a, s, &packed);
+    if (rc != FGMS_OK) return rc;
+  }
   const unsigned gx = tile_order ? (unsigned)tile_grid : (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
-  if (gx == 0) return FGMS_OK;
-  auto kern = gms_rows_kernel<T, NT, S>;
+  if (gx == 0) return a.side.kind ? launch_side_job(a.side, a.stream) : FGMS_OK;
+  auto kern = raw ? gms_rows_kernel<T, NT, S, kCanRaw> : gms_rows_kernel<T, NT, S, false>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)s.lds_rows_bytes));
@@ -707,9 +786,9 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   }
   {
     ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
-    kern<<<dim3(gx, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
+    kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
-        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1);
+        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -767,6 +846,38 @@ int pack_weights_any(const GmsArgs &a, int S, const void **packed) {
   int rc = pack_weights<float>(a, s, &p);
   *packed = p;
   return rc;
+}
+
+int planned_pack_job(const GmsArgs &a, SideJob *job, const void **packed) {
+  const Shape s = shape_of(a);
+  if (!s.ok) {
+    set_error("planned_pack_job: unsupported shape");
+    return FGMS_E_INVALID;
+  }
+  const size_t esz = a.dtype == FGMS_F16 ? 2 : 4;
+  const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+  void *ws = nullptr;
+  int rc = workspace_get(a.stream, 0, n * esz, &ws);
+  if (rc != FGMS_OK) return rc;
+  *job = SideJob{};
+  job->kind = 1;
+  job->src = a.w;
+  job->dst = ws;
+  job->n = n;
+  job->k_vol = a.k_vol; job->c_in = a.c_in; job->c_out = a.c_out;
+  job->S = s.S; job->transpose = a.transpose_w; job->dtype = a.dtype;
+  // about 8 elements per thread of 256-thread workgroups
+  size_t blocks = ((n + 2047) / 2048 + 7) / 8 * 8;
+  job->blocks = (int)(blocks > 1024 ? 1024 : blocks);
+  *packed = ws;
+  return FGMS_OK;
+}
+
+int launch_side_job(const SideJob &job, hipStream_t stream) {
+  if (job.kind == 0 || job.blocks <= 0) return FGMS_OK;
+  side_job_kernel<<<(unsigned)job.blocks, 256, 0, stream>>>(job);
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
 }
 
 bool mfma_gms_supported(const GmsArgs &a) { return shape_of(a).ok; }

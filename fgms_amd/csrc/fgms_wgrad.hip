@@ -115,7 +115,16 @@ template <typename T, int BI, int BJ>
 __global__ __launch_bounds__(kThreads) void wgrad_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap) {
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap, SideJob side) {
+  // the leading workgroups of the grid run the side job, if there is one
+  int block_x = blockIdx.x;
+  if (side.blocks) {
+    if (block_x < side.blocks) {
+      if (blockIdx.y == 0) run_side_job(side, block_x);
+      return;
+    }
+    block_x -= side.blocks;
+  }
   using W = WT<T>;
   using G = WaveGrid<BI, BJ>;
   constexpr int E = W::E, SP = W::stage_pairs, KP = W::step_pairs;
@@ -131,7 +140,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
   gs[1] = xs[1] + SP * LDI;
 
   int k, first, count;
-  if (!locate_slice(kpos, smap, k_vol, blockIdx.x, k, first, count)) return;
+  if (!locate_slice(kpos, smap, k_vol, block_x, k, first, count)) return;
   const int tiles_co = c_out / CO;
   const int ci0 = (blockIdx.y / tiles_co) * CI;
   const int co0 = (blockIdx.y % tiles_co) * CO;
@@ -270,7 +279,16 @@ template <typename T, int BI, int BJ>
 __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap) {
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap, SideJob side) {
+  // the leading workgroups of the grid run the side job, if there is one
+  int block_x = blockIdx.x;
+  if (side.blocks) {
+    if (block_x < side.blocks) {
+      if (blockIdx.y == 0) run_side_job(side, block_x);
+      return;
+    }
+    block_x -= side.blocks;
+  }
   using W = WT<T>;
   constexpr int E = W::E, SP = WTW<T>::stage_pairs, KP = W::step_pairs;
   constexpr int CI = BI * 32, CO = BJ * 32;
@@ -280,7 +298,7 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
   static_assert(NX >= 1 && NG >= 1, "stage too small");
   extern __shared__ int4v lds[];
   int k, first, count;
-  if (!locate_slice(kpos, smap, k_vol, blockIdx.x, k, first, count)) return;
+  if (!locate_slice(kpos, smap, k_vol, block_x, k, first, count)) return;
   const int tiles_co = c_out / CO;
   const int ci0 = (blockIdx.y / tiles_co) * CI;
   const int co0 = (blockIdx.y % tiles_co) * CO;
@@ -437,15 +455,10 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     }
 }
 
-// dst[i] += acc[i] rounded once to fp16, and acc[i] is reset: the accumulator is
-// handed back all-zero, which is the state the next call expects to find it in.
-template <typename T>
-__global__ void add_and_clear_kernel(T *__restrict__ dst, float *__restrict__ acc, size_t n) {
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) {
-    dst[i] = __float2half(__half2float(dst[i]) + acc[i]);
-    acc[i] = 0.f;
-  }
+// dst[i] += acc[i] rounded once to fp16 and acc[i] = 0, in a launch of its own.
+__global__ void add_and_clear_kernel(__half *__restrict__ dst, float *__restrict__ acc, size_t n) {
+  add_and_clear_elements(dst, acc, n, (size_t)blockIdx.x * blockDim.x + threadIdx.x,
+                         (size_t)gridDim.x * blockDim.x);
 }
 
 int blocks_of(int c) { return c % 128 == 0 ? 4 : (c % 64 == 0 ? 2 : 1); }
@@ -519,9 +532,9 @@ int launch(const WgradArgs &a, float *acc32) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   {
     ProfileScope prof("wgrad_kernel", a.stream);
-    kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
+    kern<<<dim3((unsigned)tiles + (unsigned)a.side.blocks, (unsigned)ty), kThreads, lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
-        a.c_out, smap);
+        a.c_out, smap, a.side);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -542,9 +555,9 @@ int launch_wave(const WgradArgs &a, float *acc32) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   {
     ProfileScope prof("wgrad_wave_kernel", a.stream);
-    kern<<<dim3((unsigned)tiles, (unsigned)ty), kThreads, lds, a.stream>>>(
+    kern<<<dim3((unsigned)tiles + (unsigned)a.side.blocks, (unsigned)ty), kThreads, lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
-        a.c_out, smap);
+        a.c_out, smap, a.side);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -587,8 +600,20 @@ int launch_mfma_wgrad(const WgradArgs &a) {
       (void)launch_fill_zero(ws, workspace_bytes(a.stream, 1), a.stream);
       return rc;
     }
-    add_and_clear_kernel<__half><<<(unsigned)((n + 255) / 256), 256, 0, a.stream>>>(
-        (__half *)a.gw, (float *)ws, n);
+    if (a.deferred_flush) {
+      // the caller attaches the flush to its next launch on the stream
+      SideJob &f = *a.deferred_flush;
+      f = SideJob{};
+      f.kind = 2;
+      f.dst = a.gw;
+      f.acc = (float *)ws;
+      f.n = n;
+      f.dtype = a.dtype;
+      size_t blocks = ((n + 2047) / 2048 + 7) / 8 * 8;   // about 8 elements per thread
+      f.blocks = (int)(blocks > 1024 ? 1024 : blocks);
+      return FGMS_OK;
+    }
+    add_and_clear_kernel<<<(unsigned)((n + 255) / 256), 256, 0, a.stream>>>((__half *)a.gw, (float *)ws, n);
     FGMS_HIP_TRY(hipGetLastError());
     return FGMS_OK;
   }

@@ -262,6 +262,28 @@ def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dty
     assert "gms_rows_kernel(fwd)" in names, names
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("shape", [(64, 64), (128, 128), (32, 64)], ids=lambda s: "%dx%d" % s)
+def test_backward_in_one_call_equals_its_two_halves(capi, shape, dtype):
+    """fgms_bwd runs the weight gradient first and lets the two main launches carry the
+    weight re-layout and the fp32 -> fp16 rounding of the weight gradient along; fgms_dgrad
+    and fgms_wgrad launch those steps by themselves.  Same input gradient bit for bit, same
+    weight gradient up to the order of its atomic sums; twice in a row, so that the fp32
+    accumulator is seen to come back empty.  (Policy 4: the kernels without atomics, also
+    where automatic dispatch would send this small scattered cloud to the pair-stationary one.)"""
+    L = layer(23, *shape, dtype)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(4)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    gi_s, gw_s = G.run_bwd(capi, D, plan=plan, split=True)
+    for _ in range(2):
+        gi_f, gw_f = G.run_bwd(capi, D, plan=plan, split=False)
+        assert np.array_equal(gi_f, gi_s)
+        G.assert_close(gw_f, gw_s, G.mode_of(L["in_feats"].dtype, False), "wgrad")
+    plan.close()
+    capi.set_kernel_policy(0)
+
+
 def test_config2_scaled_fp32_and_tf32(capi, oracle):
     L = clouds.config_case(2, scale=0.08)
     check_all(capi, oracle, L, policy=0, use_plan=True, arch80=False)
