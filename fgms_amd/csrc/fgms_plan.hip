@@ -53,7 +53,8 @@ __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
 }
 
 // One wave per block of 64 consecutive rows: which offsets have a neighbour there.
-// *stages += the number of (block, offset) combinations in use.
+// stages[0..15] together += the number of (block, offset) combinations in use (16 counters
+// so that the blocks' atomic updates do not all queue on one address).
 __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, int k_vol,
                                    unsigned long long *__restrict__ masks64, int *__restrict__ stages) {
   const int block = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
@@ -71,7 +72,7 @@ __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, 
   }
   if (threadIdx.x % 64 == 0) {
     masks64[block] = m;
-    if (m) atomicAdd(stages, __popcll(m));
+    if (m) atomicAdd(stages + (block & 15), __popcll(m));
   }
 }
 
@@ -308,13 +309,13 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       pool_alloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_cells, (size_t)4 * k_vol * p->band_count * sizeof(int32_t), s) != FGMS_OK ||
-      pool_alloc((void **)&flags, 6 * sizeof(int), s) != FGMS_OK) {
+      pool_alloc((void **)&flags, 36 * sizeof(int), s) != FGMS_OK) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
   }
   if ((rc = fill_i32(p->nbr_out, so, -1, s))) return fail(rc);
   if ((rc = fill_i32(p->nbr_in, si, -1, s))) return fail(rc);
-  if ((rc = fill_i32(flags, 6, 0, s))) return fail(rc);
+  if ((rc = fill_i32(flags, 36, 0, s))) return fail(rc);
   if (n_pairs > 0) {
     build_tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
         kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, p->nbr_out, p->nbr_in, flags);
@@ -393,7 +394,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
         tmp_tab[d] = tab;      // the unsorted table, freed after the sync
         tab = sorted;
       }
-      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask, flags + 4 + d);
+      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask, flags + 4 + 16 * d);
       // tile -> XCD homes pay off once every XCD has a few dozen tiles of its own
       static const bool xcd_homes = !(getenv("FGMS_XCD_HOME") && atoi(getenv("FGMS_XCD_HOME")) == 0);
       const int n_tiles = (int)((n + 255) / 256);
@@ -419,7 +420,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
-  int h[6] = {0, 0, 0, 0, 0, 0};
+  int h[36] = {0};
   if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
       hipStreamSynchronize(s) != hipSuccess) {
     free_tmp();
@@ -437,8 +438,11 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->fwd_ok = !h[1];
   p->dgrad_ok = !h[2];
   p->bands_ok = !h[3];
-  p->stages_out = h[4];
-  p->stages_in = h[5];
+  p->stages_out = p->stages_in = 0;
+  for (int i = 0; i < 16; ++i) {
+    p->stages_out += h[4 + i];
+    p->stages_in += h[20 + i];
+  }
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
 }
