@@ -53,10 +53,8 @@ __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
 }
 
 // One wave per block of 64 consecutive rows: which offsets have a neighbour there.
-// stages[0..15] together += the number of (block, offset) combinations in use (16 counters
-// so that the blocks' atomic updates do not all queue on one address).
 __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, int k_vol,
-                                   unsigned long long *__restrict__ masks64, int *__restrict__ stages) {
+                                   unsigned long long *__restrict__ masks64) {
   const int block = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
   const int row = block * 64 + (int)(threadIdx.x % 64);
   if (block * 64 >= n_rows) return;
@@ -70,9 +68,24 @@ __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, 
     for (int i = 0; i < 8; ++i)
       if (__ballot(g[i] >= 0)) m |= 1ull << (k0 + i);
   }
-  if (threadIdx.x % 64 == 0) {
-    masks64[block] = m;
-    if (m) atomicAdd(stages + (block & 15), __popcll(m));
+  if (threadIdx.x % 64 == 0) masks64[block] = m;
+}
+
+// *stages = the number of (block, offset) combinations in use: the set bits of all block
+// masks.  One workgroup (a few thousand masks; thousands of same-address atomics from the
+// mask kernel itself cost 25 us).
+__global__ __launch_bounds__(1024) void count_stages_kernel(const unsigned long long *__restrict__ masks64,
+                                                            int n_blocks, int *__restrict__ stages) {
+  __shared__ int partial[16];
+  int sum = 0;
+  for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) sum += __popcll(masks64[b]);
+  for (int d = 32; d > 0; d >>= 1) sum += __shfl_down(sum, d);
+  if (threadIdx.x % 64 == 0) partial[threadIdx.x / 64] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0;
+    for (int i = 0; i < (int)blockDim.x / 64; ++i) total += partial[i];
+    *stages = total;
   }
 }
 
@@ -309,13 +322,13 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       pool_alloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_cells, (size_t)4 * k_vol * p->band_count * sizeof(int32_t), s) != FGMS_OK ||
-      pool_alloc((void **)&flags, 36 * sizeof(int), s) != FGMS_OK) {
+      pool_alloc((void **)&flags, 6 * sizeof(int), s) != FGMS_OK) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
   }
   if ((rc = fill_i32(p->nbr_out, so, -1, s))) return fail(rc);
   if ((rc = fill_i32(p->nbr_in, si, -1, s))) return fail(rc);
-  if ((rc = fill_i32(flags, 36, 0, s))) return fail(rc);
+  if ((rc = fill_i32(flags, 6, 0, s))) return fail(rc);
   if (n_pairs > 0) {
     build_tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
         kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, p->nbr_out, p->nbr_in, flags);
@@ -394,7 +407,8 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
         tmp_tab[d] = tab;      // the unsorted table, freed after the sync
         tab = sorted;
       }
-      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask, flags + 4 + 16 * d);
+      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask);
+      count_stages_kernel<<<1, 1024, 0, s>>>(mask, (int)blocks, flags + 4 + d);
       // tile -> XCD homes pay off once every XCD has a few dozen tiles of its own
       static const bool xcd_homes = !(getenv("FGMS_XCD_HOME") && atoi(getenv("FGMS_XCD_HOME")) == 0);
       const int n_tiles = (int)((n + 255) / 256);
@@ -420,7 +434,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
-  int h[36] = {0};
+  int h[6] = {0, 0, 0, 0, 0, 0};
   if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
       hipStreamSynchronize(s) != hipSuccess) {
     free_tmp();
@@ -438,11 +452,8 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->fwd_ok = !h[1];
   p->dgrad_ok = !h[2];
   p->bands_ok = !h[3];
-  p->stages_out = p->stages_in = 0;
-  for (int i = 0; i < 16; ++i) {
-    p->stages_out += h[4 + i];
-    p->stages_in += h[20 + i];
-  }
+  p->stages_out = h[4];
+  p->stages_in = h[5];
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
 }
