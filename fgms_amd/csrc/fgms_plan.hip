@@ -134,7 +134,7 @@ __global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32
 //    neighbouring rows meet in one L2.
 //  * Inside an XCD the tiles are ranked by the number of offsets they use, most
 //    first: the launch lasts as long as its longest tile, so those must start
-//    first.  Ranks are laid over the CUs in a snake (round 0 forwards, round 1
+//    first.  Ranks are laid over the CUs in a snake (first sweep forwards, second
 //    backwards, ...), so every CU gets a mix of long and short tiles instead of
 //    three long ones competing for the same SIMDs.
 //  * Every XCD takes at most cap = ceil(tiles / 8) tiles; the lightest tiles of an
