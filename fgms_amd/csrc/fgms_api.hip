@@ -256,8 +256,8 @@ int check_common(const void *a, const void *b, const void *c, const int32_t *kpo
 // ones over scattered clouds qualify (256 -> 256 over a 50 k subsample: slots / pairs 2.6).
 bool sparse_rows(const GmsArgs &a, const Plan *plan) {
   const int stages = a.transpose_w ? plan->stages_in : plan->stages_out;
-  if (stages <= 0 || a.n_pairs <= 0) return false;
-  const double slots_per_pair = (double)stages * 64.0 / (double)a.n_pairs;
+  if (stages <= 0 || plan->n_pairs <= 0) return false;   // (the plan's own pair count: a.n_pairs is a bound)
+  const double slots_per_pair = (double)stages * 64.0 / (double)plan->n_pairs;
   const double c_src = a.transpose_w ? a.c_out : a.c_in;
   const double atomics = a.dtype == FGMS_F16 ? 240.0 : 64.0;
   return (c_src + atomics) * 1.15 < c_src * slots_per_pair;

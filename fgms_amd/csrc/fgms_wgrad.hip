@@ -133,11 +133,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
   constexpr int NCI = CI / E, NCO = CO / E;   // 16-byte chunks per staged row
   constexpr int NX = BI, NG = BJ;             // chunks per thread and stage
   extern __shared__ int4v lds[];
-  T *xs[2], *gs[2];
-  xs[0] = reinterpret_cast<T *>(lds);
-  gs[0] = xs[0] + SP * LDI;
-  xs[1] = gs[0] + SP * LDO;
-  gs[1] = xs[1] + SP * LDI;
+  // two staging buffers, each SP rows of `in` followed by SP rows of `dOut`.  (Addressed
+  // by arithmetic on the LDS base: through an array of pointers the compiler loses the
+  // address space and falls back to flat loads and stores, which also wait on the
+  // global loads in flight.)
+  T *const stage0 = reinterpret_cast<T *>(lds);
+  constexpr int kBufElems = SP * (LDI + LDO);
 
   int k, first, count;
   if (!locate_slice(kpos, smap, k_vol, block_x, k, first, count)) return;
@@ -159,63 +160,59 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
   int xi[NX], gi[NG];      // gather rows of the stage about to be loaded
   int4v xr[NX], gr[NG];    // its data while in flight
 
+  // Everything below is issued unconditionally and nothing touches a loaded register
+  // before its consumer: an index or a row that is selected, copied or loaded under a
+  // branch makes the compiler wait for ALL loads in flight at that point, and the row
+  // loads would no longer run under the MFMAs.  Past the end of the slice the last pair
+  // is read again; store_rows zeroes those rows by their position instead.
   auto load_idx = [&](int st) {
 #pragma unroll
-    for (int i = 0; i < NX; ++i) {
-      const int p = st * SP + (tid + kThreads * i) / NCI;
-      xi[i] = p < count ? imap[first + p] : -1;
-    }
+    for (int i = 0; i < NX; ++i)
+      xi[i] = imap[first + min(st * SP + (tid + kThreads * i) / NCI, count - 1)];
 #pragma unroll
-    for (int i = 0; i < NG; ++i) {
-      const int p = st * SP + (tid + kThreads * i) / NCO;
-      gi[i] = p < count ? omap[first + p] : -1;
-    }
+    for (int i = 0; i < NG; ++i)
+      gi[i] = omap[first + min(st * SP + (tid + kThreads * i) / NCO, count - 1)];
   };
   auto load_rows = [&]() {
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int cc = (tid + kThreads * i) % NCI;
-      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)max(xi[i], 0) * c_in + ci0 + cc * E);
+      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)xi[i] * c_in + ci0 + cc * E);
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int cc = (tid + kThreads * i) % NCO;
-      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)max(gi[i], 0) * c_out + co0 + cc * E);
+      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
     }
-#pragma unroll
-    for (int i = 0; i < NX; ++i)
-      if (xi[i] < 0) xr[i] = int4v{0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < NG; ++i)
-      if (gi[i] < 0) gr[i] = int4v{0, 0, 0, 0};
   };
-  auto store_rows = [&](int buf) {
+  auto store_rows = [&](int buf, int st) {   // st: the stage the rows in flight belong to
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int e = tid + kThreads * i;
-      *reinterpret_cast<int4v *>(xs[buf] + (e / NCI) * LDI + (e % NCI) * E) = xr[i];
+      *reinterpret_cast<int4v *>(stage0 + buf * kBufElems + (e / NCI) * LDI + (e % NCI) * E) =
+          st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int e = tid + kThreads * i;
-      *reinterpret_cast<int4v *>(gs[buf] + (e / NCO) * LDO + (e % NCO) * E) = gr[i];
+      *reinterpret_cast<int4v *>(stage0 + buf * kBufElems + SP * LDI + (e / NCO) * LDO + (e % NCO) * E) =
+          st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
     }
   };
 
   load_idx(0);
   load_rows();
-  store_rows(0);
-  if (nstages > 1) load_idx(1);
+  store_rows(0, 0);
+  load_idx(1);
   __syncthreads();
 
   for (int st = 0; st < nstages; ++st) {
     const int cur = st & 1;
-    const bool more = st + 1 < nstages;
-    if (more) {
-      load_rows();                          // stage st + 1, in flight during the MFMAs
-      if (st + 2 < nstages) load_idx(st + 2);
-    }
-    const T *x = xs[cur], *g = gs[cur];
+    load_rows();                            // stage st + 1, in flight during the MFMAs
+    __builtin_amdgcn_sched_barrier(0);      // (rows first, then indices, both before the MFMAs)
+    load_idx(st + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    const T *x = stage0 + cur * kBufElems, *g = x + SP * LDI;
 #pragma unroll
     for (int ks = wk; ks < SP / KP; ks += G::WK) {
       const int p0 = ks * KP;
@@ -247,7 +244,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
         }
       }
     }
-    if (more) store_rows(cur ^ 1);
+    // the stores wait for the rows in flight: keep them (and that wait) behind the MFMAs
+    __builtin_amdgcn_sched_barrier(0);
+    store_rows(cur ^ 1, st + 1);
     __syncthreads();
   }
 
@@ -316,47 +315,45 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
 
   const int nstages = (count + SP - 1) / SP;
   int xi[NX], gi[NG];        // gather rows of the next stage to load
-  int xs[NX], gs[NG];        // ... of the stage in flight (sign = padding row)
-  int4v xr[NX], gr[NG];      // its data
+  int4v xr[NX], gr[NG];      // the rows in flight
 
+  // Everything is issued unconditionally and nothing touches a loaded register before
+  // its consumer: an index or a row that is selected, copied or loaded under a branch
+  // makes the compiler wait for ALL loads in flight at that point, and the row loads
+  // would no longer run under the MFMAs.  Past the end of the slice the last pair is
+  // read again; store_rows zeroes those rows by their position instead.
   auto load_idx = [&](int st) {
 #pragma unroll
-    for (int i = 0; i < NX; ++i) {
-      const int p = st * SP + (lane + 64 * i) / NCI;
-      xi[i] = p < count ? imap[first + p] : -1;
-    }
+    for (int i = 0; i < NX; ++i)
+      xi[i] = imap[first + min(st * SP + (lane + 64 * i) / NCI, count - 1)];
 #pragma unroll
-    for (int i = 0; i < NG; ++i) {
-      const int p = st * SP + (lane + 64 * i) / NCO;
-      gi[i] = p < count ? omap[first + p] : -1;
-    }
+    for (int i = 0; i < NG; ++i)
+      gi[i] = omap[first + min(st * SP + (lane + 64 * i) / NCO, count - 1)];
   };
   auto load_rows = [&]() {
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int cc = (lane + 64 * i) % NCI;
-      xs[i] = xi[i];
-      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)max(xi[i], 0) * c_in + ci0 + cc * E);
+      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)xi[i] * c_in + ci0 + cc * E);
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int cc = (lane + 64 * i) % NCO;
-      gs[i] = gi[i];
-      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)max(gi[i], 0) * c_out + co0 + cc * E);
+      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
     }
   };
-  auto store_rows = [&]() {
+  auto store_rows = [&](int st) {     // st: the stage the rows in flight belong to
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int e = lane + 64 * i;
       *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
-          xs[i] < 0 ? int4v{0, 0, 0, 0} : xr[i];
+          st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int e = lane + 64 * i;
       *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
-          gs[i] < 0 ? int4v{0, 0, 0, 0} : gr[i];
+          st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
     }
   };
   auto wave_fence = [] {
@@ -365,19 +362,16 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
   };
 
   int st = wave;
-  if (st < nstages) {
-    load_idx(st);
-    load_rows();
-    if (st + 4 < nstages) load_idx(st + 4);
-  }
+  load_idx(st);
+  load_rows();
+  load_idx(st + 4);
   while (st < nstages) {
-    store_rows();                   // waits for the stage's rows
+    store_rows(st);                 // waits for the stage's rows
     wave_fence();
-    const int nxt = st + 4;
-    if (nxt < nstages) {
-      load_rows();                  // next stage, in flight during the MFMAs
-      if (nxt + 4 < nstages) load_idx(nxt + 4);
-    }
+    load_rows();                    // stage st + 4, in flight during the MFMAs
+    __builtin_amdgcn_sched_barrier(0);   // (rows first, then indices, both before the MFMAs:
+    load_idx(st + 8);                    //  the wait for the rows then leaves the indices in flight)
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < SP / KP; ++ks) {
       const int p0 = ks * KP;
@@ -410,7 +404,7 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
       }
     }
     wave_fence();                   // the tile is rewritten at the top of the loop
-    st = nxt;
+    st += 4;
   }
 
   // sum the four waves' tiles: (2, 3) -> (0, 1), then 1 -> 0, through LDS
