@@ -81,35 +81,6 @@ __device__ __forceinline__ void load_weights(int4v *__restrict__ w_lds,
   }
 }
 
-// Gathers one slab of the wave's 64 rows into its LDS staging tile.
-template <typename T, int S>
-__device__ __forceinline__ void stage_rows(int4v *__restrict__ a_lds, const int *__restrict__ idx,
-                                           const T *__restrict__ src, int c_src, int slab,
-                                           int lane) {
-  constexpr int E = Elem<T>::per_chunk;
-  constexpr int C = 2 * S;
-  int4v v[C];
-  int g[C];
-#pragma unroll
-  for (int it = 0; it < C; ++it) g[it] = idx[(it * 64 + lane) / C];
-  // every lane loads (absent rows read row 0 and are zeroed afterwards): no
-  // branch between the loads, so all of them are in flight together
-#pragma unroll
-  for (int it = 0; it < C; ++it) {
-    const int c = (it * 64 + lane) % C;
-    v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(g[it], 0) * c_src +
-                                             (size_t)(slab * C + c) * E);
-  }
-#pragma unroll
-  for (int it = 0; it < C; ++it)
-    if (g[it] < 0) v[it] = int4v{0, 0, 0, 0};
-#pragma unroll
-  for (int it = 0; it < C; ++it) {
-    const int slot = it * 64 + lane;
-    a_lds[a_slot<S>(slot / C, slot % C)] = v[it];
-  }
-}
-
 // acc[mt][nt] += A(slab) x W(slab).
 template <typename T, int NT, int S>
 __device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
@@ -375,6 +346,38 @@ __device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__
 }
 
 // ---------------------------------------------------------------------------
+// Row gathers in two steps, so that the loads of one slab run under the MFMAs of the
+// previous one: issue (global -> registers, absent rows read row 0) and commit
+// (registers -> the wave's LDS tile, absent rows as zeros; waits for the loads).
+template <typename T, int S>
+__device__ __forceinline__ void gather_issue(int4v (&v)[2 * S], int (&g)[2 * S],
+                                             const int *__restrict__ idx,
+                                             const T *__restrict__ src, int c_src, int slab,
+                                             int lane) {
+  constexpr int E = Elem<T>::per_chunk;
+  constexpr int C = 2 * S;
+#pragma unroll
+  for (int it = 0; it < C; ++it) g[it] = idx[(it * 64 + lane) / C];
+#pragma unroll
+  for (int it = 0; it < C; ++it) {
+    const int c = (it * 64 + lane) % C;
+    v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(g[it], 0) * c_src +
+                                             (size_t)(slab * C + c) * E);
+  }
+}
+
+template <int S>
+__device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (&v)[2 * S],
+                                              const int (&g)[2 * S], int lane) {
+  constexpr int C = 2 * S;
+#pragma unroll
+  for (int it = 0; it < C; ++it) {
+    const int slot = it * 64 + lane;
+    a_lds[a_slot<S>(slot / C, slot % C)] = g[it] < 0 ? int4v{0, 0, 0, 0} : v[it];
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Pair-stationary kernel.
 template <typename T, int NT, int S>
 __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
@@ -431,9 +434,13 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
 
+    int4v v[2 * S];
+    int gsel[2 * S];
+    gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
     for (int slab = 0; slab < slabs; ++slab) {
-      stage_rows<T, S>(a_lds, gidx, src, c_src, slab, lane);
+      gather_commit<S>(a_lds, v, gsel, lane);
       wave_lds_fence();
+      if (slab + 1 < slabs) gather_issue<T, S>(v, gsel, gidx, src, c_src, slab + 1, lane);   // under the MFMAs
       mma_slab<T, NT, S>(acc, a_lds, w_lds, slab, lane);
       wave_lds_fence();
     }
@@ -453,34 +460,6 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 // written to LDS after the MFMAs and one barrier closes the stage.  Weights are
 // double-buffered in LDS, each wave's row tile is single-buffered (only its own
 // wave reads it).
-template <typename T, int S>
-__device__ __forceinline__ void gather_issue(int4v (&v)[2 * S], int (&g)[2 * S],
-                                             const int *__restrict__ idx,
-                                             const T *__restrict__ src, int c_src, int slab,
-                                             int lane) {
-  constexpr int E = Elem<T>::per_chunk;
-  constexpr int C = 2 * S;
-#pragma unroll
-  for (int it = 0; it < C; ++it) g[it] = idx[(it * 64 + lane) / C];
-#pragma unroll
-  for (int it = 0; it < C; ++it) {
-    const int c = (it * 64 + lane) % C;
-    v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(g[it], 0) * c_src +
-                                             (size_t)(slab * C + c) * E);
-  }
-}
-
-template <int S>
-__device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (&v)[2 * S],
-                                              const int (&g)[2 * S], int lane) {
-  constexpr int C = 2 * S;
-#pragma unroll
-  for (int it = 0; it < C; ++it) {
-    const int slot = it * 64 + lane;
-    a_lds[a_slot<S>(slot / C, slot % C)] = g[it] < 0 ? int4v{0, 0, 0, 0} : v[it];
-  }
-}
-
 // RAW: `packed` is the caller's weight tensor itself (forward, fp16: see raw_weight_frag);
 // otherwise the re-laid copy pack_weight_elements makes.
 template <typename T, int NT, int S, bool RAW>
