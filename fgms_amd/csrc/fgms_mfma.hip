@@ -483,6 +483,9 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   constexpr int NW = (WCH + kThreads - 1) / kThreads;     // ... per thread
   extern __shared__ int4v lds[];
   __shared__ unsigned long long wg_mask;
+  // fp32 only: its MFMA phase is long enough (4 k clocks a stage) to absorb the loads'
+  // issue waits; for fp16 the interleaved stage measured 2 us slower per launch
+  constexpr bool kInterleave = sizeof(T) == 4;
   const int slabs = c_src / (C * E);
   const int nts = c_dst / 32;
   int4v *w_lds = lds;                                     // [2][WCH]
@@ -613,12 +616,46 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
         gidx[lane] = g_nxt;
         wave_lds_fence();
       }
-      weights_issue(wreg, nk, nslab);
-      if (next_active) gather_issue<T, S>(v, gsel, gidx, src, c_src, nslab, lane);
     }
-    if (active) {
-      if constexpr (RAW) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
-      else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+    if (kInterleave && has_next && active && next_active) {
+      // The common stage: this stage's MFMAs with the next stage's loads between them,
+      // one row load after each (k-step, row tile) group.  A load instruction waits at
+      // issue while the CU's memory queue is full; issued in a block before the MFMAs
+      // those waits come on top of the MFMA time, issued between them they pass while
+      // the matrix pipe works off what it has.  (MFMAs and loads stay on their side of
+      // each scheduling barrier, LDS reads and address arithmetic may cross.)
+      const int4v *wl = w_lds + buf * WCH;
+      const int h = lane / 32, r = lane % 32;
+      weights_issue(wreg, nk, nslab);
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+        int4v b[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          if constexpr (RAW) b[nt] = raw_weight_frag<NT, S>(wl, s, nt, lane);
+          else b[nt] = wl[(s * NT + nt) * 64 + lane];
+        }
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+          const int it = s * 2 + mt;                       // one of the C = 2 * S row loads
+          gsel[it] = gidx[(it * 64 + lane) / C];
+          v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(gsel[it], 0) * c_src +
+                                                   (size_t)(nslab * C + (it * 64 + lane) % C) * E);
+          __builtin_amdgcn_sched_barrier(0x386);
+        }
+      }
+    } else {
+      if (has_next) {
+        weights_issue(wreg, nk, nslab);
+        if (next_active) gather_issue<T, S>(v, gsel, gidx, src, c_src, nslab, lane);
+      }
+      if (active) {
+        if constexpr (RAW) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+        else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+      }
     }
     if (!has_next) break;
     wave_lds_fence();
