@@ -100,3 +100,41 @@ def test_config1_full_size_against_oracle(capi, oracle):
     G.assert_close(gi.cpu().numpy(), oracle.c_dgrad(L["out_grad"], L["kernel"], *a, L["n_in"]), "fp32", "dgrad")
     G.assert_close(gw.cpu().numpy(), oracle.c_wgrad(L["in_feats"], L["out_grad"], *a, L["k_vol"]), "fp32", "wgrad")
     plan.close()
+
+
+@pytest.mark.parametrize("side,c,dtype,tol", [(100, 64, torch.float16, 2e-3), (96, 32, torch.float32, 2e-5)],
+                         ids=["1M-fp16", "885k-fp32"])
+def test_dense_grid_built_and_convolved_on_the_device(capi, side, c, dtype, tol):
+    """A full side^3 grid (every voxel has all its in-grid neighbours): the map comes from
+    the device builder and its size has a closed form, sum over offsets of
+    (side-|dx|)(side-|dy|)(side-|dz|); the three kernels must agree on the trilinear form at
+    a size (26 M pairs) far beyond the oracle's reach."""
+    n = side ** 3
+    g = torch.arange(side, dtype=torch.int32, device="cuda")
+    coords = torch.stack(torch.meshgrid(g, g, g, indexing="ij"), -1).reshape(-1, 3).contiguous()
+    offs = np.array([(a, b, d) for a in (-1, 0, 1) for b in (-1, 0, 1) for d in (-1, 0, 1)], np.int32)
+    imap, omap, knnz, kpos = capi.build_kernel_map(coords, coords, offs, 1)
+    expect = [(side - abs(a)) * (side - abs(b)) * (side - abs(d)) for a, b, d in offs]
+    assert [int(v) for v in knnz] == expect and int(imap.numel()) == sum(expect)
+    gen = torch.Generator(device="cuda").manual_seed(side)
+    x = torch.randn(n, c, device="cuda", dtype=dtype, generator=gen)
+    w = (torch.randn(27, c, c, device="cuda", generator=gen) * 0.05).to(dtype)
+    go = torch.randn(n, c, device="cuda", dtype=dtype, generator=gen)
+    plan = capi.Plan(kpos, imap, omap, n, n)
+    out = torch.zeros(n, c, device="cuda", dtype=dtype)
+    gi, gw = torch.zeros_like(x), torch.zeros_like(w)
+    capi.fusion_fwd(x, w, 0, out, kpos, None, imap, omap, False, False, plan=plan)
+    capi.bwd(go, x, w, 0, gi, gw, kpos, None, imap, omap, False, False, plan=plan)
+    torch.cuda.synchronize()
+    t_f, t_d, t_w = dot(go, out), dot(gi, x), dot(gw, w)
+    scale = float(out.double().norm() * go.double().norm())
+    assert abs(t_f - t_d) <= tol * scale and abs(t_f - t_w) <= tol * scale, (t_f, t_d, t_w, scale)
+    # an interior voxel against the definition: sum over offsets of x[neighbour] @ w[k]
+    v = (side // 2 * side + side // 2) * side + side // 2
+    ref = torch.zeros(c, dtype=torch.float64, device="cuda")
+    for k, (a, b, d) in enumerate(offs):
+        u = v + (int(a) * side + int(b)) * side + int(d)
+        ref += x[u].double() @ w[k].double()
+    assert torch.allclose(out[v].double(), ref, rtol=1e-2 if dtype == torch.float16 else 1e-5,
+                          atol=1e-2 if dtype == torch.float16 else 1e-5)
+    plan.close()
