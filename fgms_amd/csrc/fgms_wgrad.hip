@@ -18,6 +18,8 @@
 // per lane, so plain ds_read_b32 along a row is already the right shape.
 #include <type_traits>
 
+#include <stdlib.h>
+
 #include "fgms_device.h"
 #include "fgms_internal.h"
 
@@ -28,9 +30,11 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
+constexpr int kSkinnyThreads = 256;    // the skinny weight-gradient kernel
 
 template <typename T> struct WT;
 template <> struct WT<__half> {
@@ -449,6 +453,172 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Skinny layers (4 / 8 / 16 input channels, e.g. the 4 -> 32 first layer of a voxel
+// network): a 4 x 32 tile of dW[k] is no work for the matrix cores and the pass is all
+// gathers, 8 + 64 bytes a pair in fp16 -- so few bytes per pair that the number of load
+// INSTRUCTIONS is what counts.  A wave takes 64 pairs a round: lane l fetches the two
+// indices and the whole input row of pair l (one instruction each for the wave), then the
+// round is worked off in U steps of 64 / U pairs, GD = U lanes sharing a pair with 16 bytes
+// of its output-gradient row each (one load instruction a step); the pair's index and
+// input row reach those lanes by shuffles.  A lane keeps a CS x KD block of products in
+// registers.  Everything is loaded unconditionally (clamped to the slice; pairs past its
+// end count with weight 0).  At the end the lanes that hold the same channels add up
+// (shuffles), then the four waves (LDS), then one atomic add per tile element and
+// workgroup.
+// N consecutive elements (a multiple of four; 8- or 16-byte aligned) widened to fp32.
+template <typename T, int N>
+__device__ __forceinline__ void load_elems(float (&x)[N], const T *__restrict__ p) {
+  static_assert(N % 4 == 0, "rows are read four elements at a time");
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i) {
+      const float4v v = reinterpret_cast<const float4v *>(p)[i];
+      x[4 * i] = v[0]; x[4 * i + 1] = v[1]; x[4 * i + 2] = v[2]; x[4 * i + 3] = v[3];
+    }
+  } else if constexpr (N % 8 == 0) {
+#pragma unroll
+    for (int i = 0; i < N / 8; ++i) {
+      const half8 v = reinterpret_cast<const half8 *>(p)[i];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[8 * i + j] = (float)v[j];
+    }
+  } else {
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i) {
+      const half4 v = reinterpret_cast<const half4 *>(p)[i];
+      x[4 * i] = (float)v[0]; x[4 * i + 1] = (float)v[1]; x[4 * i + 2] = (float)v[2]; x[4 * i + 3] = (float)v[3];
+    }
+  }
+}
+
+template <typename T, int CS, int CD>
+__global__ __launch_bounds__(kSkinnyThreads) void wgrad_skinny_kernel(
+    const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
+    const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+    const int32_t *__restrict__ omap, int k_vol, SliceMap smap) {
+  constexpr int KD = 16 / (int)sizeof(T);     // output channels per lane: one 16-byte load
+  constexpr int GD = CD / KD;                 // lanes per pair = steps per round
+  constexpr int PPS = 64 / GD;                // pairs per step
+  constexpr int XW = CS * (int)sizeof(T) / 4; // 32-bit words of an input row
+  static_assert(CD % KD == 0 && 64 % GD == 0 && XW >= 1, "shape");
+  extern __shared__ float red[];            // [waves - 1][CS][CD]
+  constexpr int kWavesS = kSkinnyThreads / 64;
+  int k, first, count;
+  if (!locate_slice(kpos, smap, k_vol, blockIdx.x, k, first, count)) return;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int sub = lane / GD, cg = lane % GD;
+  const int rounds = (count + kSkinnyThreads - 1) / kSkinnyThreads;
+
+  float acc[CS][KD];
+#pragma unroll
+  for (int i = 0; i < CS; ++i)
+#pragma unroll
+    for (int j = 0; j < KD; ++j) acc[i][j] = 0.f;
+
+  // pair lane l fetches in round rd
+  auto my_pair = [&](int rd) { return (rd * kWavesS + wave) * 64 + lane; };
+  auto load_x = [&](uint32_t (&xw)[XW], int row) {
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(in + (size_t)row * CS);
+    if constexpr (XW % 4 == 0) {
+#pragma unroll
+      for (int i = 0; i < XW / 4; ++i) {
+        const int4v v = reinterpret_cast<const int4v *>(p)[i];
+        xw[4 * i] = v[0]; xw[4 * i + 1] = v[1]; xw[4 * i + 2] = v[2]; xw[4 * i + 3] = v[3];
+      }
+    } else {
+      typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int i = 0; i < XW / 2; ++i) {
+        const uint2v v = reinterpret_cast<const uint2v *>(p)[i];
+        xw[2 * i] = v[0]; xw[2 * i + 1] = v[1];
+      }
+    }
+  };
+  // Pipeline over the rounds: entering round rd the input rows and output-gradient rows
+  // of rd and the indices of rd + 1 are there (or on their way); the round issues the
+  // indices of rd + 2 and the rows of rd + 1 in one block, then multiplies.  The
+  // scheduling barrier keeps the loads together in front of the arithmetic (left alone,
+  // the compiler feeds them in one at a time between the multiply-adds, each waiting for
+  // the one before).
+  auto load_g = [&](float (&g)[GD][KD], int gi_lane) {
+#pragma unroll
+    for (int u = 0; u < GD; ++u) {
+      const int row = __shfl(gi_lane, u * PPS + sub);
+      load_elems<T, KD>(g[u], gout + (size_t)row * CD + cg * KD);
+    }
+  };
+  uint32_t xw[XW], xw_n[XW];
+  float g[GD][KD], g_n[GD][KD];
+  {
+    const int p0 = first + min(my_pair(0), count - 1);
+    load_x(xw, imap[p0]);
+    load_g(g, omap[p0]);
+  }
+  int xi_n = imap[first + min(my_pair(1), count - 1)], gi_n = omap[first + min(my_pair(1), count - 1)];
+  for (int rd = 0; rd < rounds; ++rd) {
+    const int p_nn = first + min(my_pair(rd + 2), count - 1);
+    const int xi_nn = imap[p_nn], gi_nn = omap[p_nn];
+    load_x(xw_n, xi_n);
+    load_g(g_n, gi_n);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < GD; ++u) {
+      const int src = u * PPS + sub;
+      const float live = (rd * kWavesS + wave) * 64 + src < count ? 1.f : 0.f;
+      float x[CS];
+#pragma unroll
+      for (int i = 0; i < XW; ++i) {
+        const uint32_t word = (uint32_t)__shfl((int)xw[i], src);
+        if constexpr (sizeof(T) == 4) {
+          x[i] = __builtin_bit_cast(float, word) * live;
+        } else {
+          x[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(word & 0xffffu)) * live;
+          x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(word >> 16)) * live;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < CS; ++i)
+#pragma unroll
+        for (int j = 0; j < KD; ++j) acc[i][j] += x[i] * g[u][j];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < XW; ++i) xw[i] = xw_n[i];
+#pragma unroll
+    for (int u = 0; u < GD; ++u)
+#pragma unroll
+      for (int j = 0; j < KD; ++j) g[u][j] = g_n[u][j];
+    xi_n = xi_nn;
+    gi_n = gi_nn;
+  }
+  // lanes sub = 0 .. PPS-1 with the same cg hold the same channels
+#pragma unroll
+  for (int off = GD; off < 64; off <<= 1)
+#pragma unroll
+    for (int i = 0; i < CS; ++i)
+#pragma unroll
+      for (int j = 0; j < KD; ++j) acc[i][j] += __shfl_xor(acc[i][j], off);
+  if (wave > 0 && sub == 0) {
+#pragma unroll
+    for (int i = 0; i < CS; ++i)
+#pragma unroll
+      for (int j = 0; j < KD; ++j) red[((wave - 1) * CS + i) * CD + cg * KD + j] = acc[i][j];
+  }
+  __syncthreads();
+  if (wave == 0 && sub == 0) {
+#pragma unroll
+    for (int i = 0; i < CS; ++i)
+#pragma unroll
+      for (int j = 0; j < KD; ++j) {
+        float v = acc[i][j];
+        for (int w = 0; w < kWavesS - 1; ++w) v += red[(w * CS + i) * CD + cg * KD + j];
+        atomic_add(gw32 + ((size_t)k * CS + i) * CD + cg * KD + j, v);
+      }
+  }
+}
+
 // dst[i] += acc[i] rounded once to fp16 and acc[i] = 0, in a launch of its own.
 __global__ void add_and_clear_kernel(__half *__restrict__ dst, float *__restrict__ acc, size_t n) {
   add_and_clear_elements(dst, acc, n, (size_t)blockIdx.x * blockDim.x + threadIdx.x,
@@ -557,8 +727,49 @@ int launch_wave(const WgradArgs &a, float *acc32) {
   return FGMS_OK;
 }
 
+bool skinny_shape(const WgradArgs &a) {
+  const size_t esz = a.dtype == FGMS_F16 ? 2 : 4;
+  return (a.c_in == 4 || a.c_in == 8 || a.c_in == 16) && (a.c_out == 16 || a.c_out == 32 || a.c_out == 64) &&
+         reinterpret_cast<uintptr_t>(a.in) % 16 == 0 && reinterpret_cast<uintptr_t>(a.gout) % 16 == 0 &&
+         (size_t)a.c_in * esz % 8 == 0;
+}
+
+template <typename T, int CS, int CD>
+int launch_skinny(const WgradArgs &a, float *acc32) {
+  if (a.side.kind != 0) {       // nothing rides along with this launch
+    int rc = launch_side_job(a.side, a.stream);
+    if (rc != FGMS_OK) return rc;
+  }
+  // Few, big workgroups (about two to a CU): measured on the 4 -> 32 layer over 2.1 M
+  // pairs, 34 us against 40 us with six to a CU, 36-72 us with equal runs of the pair list
+  // instead of the plan's (offset, band) cells (workgroups that run at the same time then
+  // work on the same offset and their closing atomic adds queue on the same addresses),
+  // and 40-68 us with 16-wave workgroups.
+  static const int wgs_per_cu = getenv("FGMS_SKINNY_WGS") ? atoi(getenv("FGMS_SKINNY_WGS")) : 2;
+  const SliceMap smap = choose_slices(a, 1, 64, (int64_t)num_cus() * wgs_per_cu);
+  const int64_t tiles = (int64_t)smap.slices * a.k_vol;
+  const size_t lds = (size_t)(kSkinnyThreads / 64 - 1) * CS * CD * sizeof(float);
+  auto kern = wgrad_skinny_kernel<T, CS, CD>;
+  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  {
+    ProfileScope prof("wgrad_skinny_kernel", a.stream);
+    kern<<<(unsigned)tiles, kSkinnyThreads, lds, a.stream>>>(
+        (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, smap);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
 template <typename T>
 int dispatch(const WgradArgs &a, float *acc32) {
+  if (skinny_shape(a)) {
+#define FGMS_WS(I, J) if (a.c_in == I && a.c_out == J) return launch_skinny<T, I, J>(a, acc32);
+    FGMS_WS(4, 16) FGMS_WS(4, 32) FGMS_WS(4, 64)
+    FGMS_WS(8, 16) FGMS_WS(8, 32) FGMS_WS(8, 64)
+    FGMS_WS(16, 16) FGMS_WS(16, 32) FGMS_WS(16, 64)
+#undef FGMS_WS
+  }
   const int bi = blocks_of(a.c_in), bj = blocks_of(a.c_out);
 #define FGMS_WW(I, J) if (bi == I && bj == J) return launch_wave<T, I, J>(a, acc32);
   FGMS_WW(1, 1) FGMS_WW(1, 2) FGMS_WW(2, 1) FGMS_WW(2, 2)
@@ -574,6 +785,7 @@ int dispatch(const WgradArgs &a, float *acc32) {
 }  // namespace
 
 bool mfma_wgrad_supported(const WgradArgs &a) {
+  if (skinny_shape(a)) return true;     // (no MFMA there: the skinny kernel shares this path's accumulator)
   if (a.c_in % 32 != 0 || a.c_out % 32 != 0) return false;
   if (reinterpret_cast<uintptr_t>(a.in) % 16 || reinterpret_cast<uintptr_t>(a.gout) % 16) return false;
   return true;

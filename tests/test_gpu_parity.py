@@ -101,6 +101,16 @@ def test_skinny_layers_by_waves_per_block(capi, oracle, monkeypatch, shape, part
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("use_plan", [True, False], ids=["plan", "noplan"])
+@pytest.mark.parametrize("shape", [(4, 16), (4, 64), (8, 32), (16, 64), (16, 16)], ids=lambda s: "%dx%d" % s)
+def test_skinny_weight_gradient_shapes(capi, oracle, shape, use_plan, dtype):
+    """Layers with 4 / 8 / 16 input channels: forward, input gradient and the skinny
+    weight-gradient kernel (lanes share a pair, four output channels each), sliced by the
+    plan's row bands or, without a plan, by pair count."""
+    check_all(capi, oracle, layer(29, *shape, dtype), policy=0, use_plan=use_plan)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
 @pytest.mark.parametrize("kind,shape", [("down", (64, 128)), ("up", (128, 64)), ("down", (16, 32)), ("up", (5, 3))])
 def test_strided_and_transposed(capi, oracle, kind, shape, dtype):
     L = layer(14, shape[0], shape[1], dtype, kind)
