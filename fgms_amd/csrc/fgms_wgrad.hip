@@ -161,14 +161,17 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   const int nstages = (count + SP - 1) / SP;
-  int xi[NX], gi[NG];      // gather rows of the stage about to be loaded
-  int4v xr[NX], gr[NG];    // its data while in flight
+  int xi[NX], gi[NG];                  // gather rows of the stage about to be loaded
+  int4v xa[NX], ga[NG], xb[NX], gb[NG];  // rows in flight: even stages in (xa, ga), odd ones in (xb, gb)
 
   // Everything below is issued unconditionally and nothing touches a loaded register
   // before its consumer: an index or a row that is selected, copied or loaded under a
   // branch makes the compiler wait for ALL loads in flight at that point, and the row
   // loads would no longer run under the MFMAs.  Past the end of the slice the last pair
   // is read again; store_rows zeroes those rows by their position instead.
+  // Two stages of rows are in flight: loads complete in order, so the indices of stage
+  // s + 1 are issued BEFORE the rows of stage s -- waiting for those indices then leaves
+  // the rows behind them in flight.
   auto load_idx = [&](int st) {
 #pragma unroll
     for (int i = 0; i < NX; ++i)
@@ -177,19 +180,19 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
     for (int i = 0; i < NG; ++i)
       gi[i] = omap[first + min(st * SP + (tid + kThreads * i) / NCO, count - 1)];
   };
-  auto load_rows = [&]() {
+  auto load_rows = [&](int4v (&xr)[NX], int4v (&gr)[NG], const int (&xrow)[NX], const int (&grow)[NG]) {
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int cc = (tid + kThreads * i) % NCI;
-      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)xi[i] * c_in + ci0 + cc * E);
+      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)xrow[i] * c_in + ci0 + cc * E);
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int cc = (tid + kThreads * i) % NCO;
-      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
+      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)grow[i] * c_out + co0 + cc * E);
     }
   };
-  auto store_rows = [&](int buf, int st) {   // st: the stage the rows in flight belong to
+  auto store_rows = [&](int buf, int st, const int4v (&xr)[NX], const int4v (&gr)[NG]) {
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int e = tid + kThreads * i;
@@ -203,19 +206,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
           st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
     }
   };
-
-  load_idx(0);
-  load_rows();
-  store_rows(0, 0);
-  load_idx(1);
-  __syncthreads();
-
-  for (int st = 0; st < nstages; ++st) {
-    const int cur = st & 1;
-    load_rows();                            // stage st + 1, in flight during the MFMAs
-    __builtin_amdgcn_sched_barrier(0);      // (rows first, then indices, both before the MFMAs)
-    load_idx(st + 2);
-    __builtin_amdgcn_sched_barrier(0);
+  auto multiply = [&](int cur) {
     const T *x = stage0 + cur * kBufElems, *g = x + SP * LDI;
 #pragma unroll
     for (int ks = wk; ks < SP / KP; ks += G::WK) {
@@ -248,10 +239,52 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
         }
       }
     }
-    // the stores wait for the rows in flight: keep them (and that wait) behind the MFMAs
+  };
+  // one stage: LDS buffer `cur` holds stage st; the rows of st + 1 are in flight in
+  // (xn, gn), the index registers hold stage st + 2; (xf, gf) is free
+  auto stage = [&](int st, int cur, int4v (&xf)[NX], int4v (&gf)[NG], const int4v (&xn)[NX],
+                   const int4v (&gn)[NG]) {
+    int xrow[NX], grow[NG];
+#pragma unroll
+    for (int i = 0; i < NX; ++i) xrow[i] = xi[i];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) grow[i] = gi[i];
+    load_idx(st + 3);                       // indices first ...
     __builtin_amdgcn_sched_barrier(0);
-    store_rows(cur ^ 1, st + 1);
+    load_rows(xf, gf, xrow, grow);          // ... then the rows of stage st + 2
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(cur);
+    // the stores wait for the rows of st + 1: keep them (and that wait) behind the MFMAs
+    __builtin_amdgcn_sched_barrier(0);
+    store_rows(cur ^ 1, st + 1, xn, gn);
     __syncthreads();
+  };
+
+  load_idx(0);
+  {
+    int xrow[NX], grow[NG];
+#pragma unroll
+    for (int i = 0; i < NX; ++i) xrow[i] = xi[i];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) grow[i] = gi[i];
+    load_idx(1);
+    load_rows(xa, ga, xrow, grow);          // stage 0
+  }
+  {
+    int xrow[NX], grow[NG];
+#pragma unroll
+    for (int i = 0; i < NX; ++i) xrow[i] = xi[i];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) grow[i] = gi[i];
+    load_idx(2);
+    load_rows(xb, gb, xrow, grow);          // stage 1
+  }
+  store_rows(0, 0, xa, ga);
+  __syncthreads();
+  for (int st = 0; st < nstages; st += 2) {
+    stage(st, 0, xa, ga, xb, gb);
+    if (st + 1 >= nstages) break;
+    stage(st + 1, 1, xb, gb, xa, ga);
   }
 
   // flush: accumulator register r of lane l is row (r/4)*8 + (l/32)*4 + r%4, column l%32
