@@ -90,9 +90,26 @@ def build_torch_ext(verbose=False):
     return out
 
 
+DEMO_PATH = os.path.join(LIB_DIR, "cabi_demo")
+
+
+def build_cabi_demo(verbose=False):
+    """tests/cabi_demo.c: a plain C program over include/fgms.h (host code only)."""
+    cmd = [os.environ.get("CC", "gcc"), "-O2", "-std=c11", "-D__HIP_PLATFORM_AMD__=1",
+           "-I", "/opt/rocm/include", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cabi_demo.c"), "-o", DEMO_PATH,
+           "-L", LIB_DIR, "-lfgms_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
+    o = _run(cmd)
+    if verbose and o.strip():
+        print(o)
+    return DEMO_PATH
+
+
 def build_all(verbose=False):
     build_hip_lib(verbose)
     build_torch_ext(verbose)
+    build_cabi_demo(verbose)
 
 
 if __name__ == "__main__":
