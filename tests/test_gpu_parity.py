@@ -259,6 +259,22 @@ def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dty
     ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
     G.assert_close(out, ref, G.mode_of(L["in_feats"].dtype, False), "fwd")
 
+    # policy 4 keeps the scattered layer on the output-stationary kernel: same bits every run
+    capi.set_kernel_policy(4)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    capi.profile_enable(True)
+    first = G.run_fwd(capi, D, fused=True, plan=plan)
+    second = G.run_fwd(capi, D, fused=True, plan=plan)
+    torch.cuda.synchronize()
+    capi.profile_enable(False)
+    names = [n for n, _ in capi.profile_records()]
+    capi.profile_reset()
+    plan.close()
+    capi.set_kernel_policy(0)
+    assert "gms_rows_kernel(fwd)" in names and "gms_pairs_kernel(fwd)" not in names, names
+    assert np.array_equal(first, second)
+    G.assert_close(first, ref, G.mode_of(L["in_feats"].dtype, False), "fwd, policy 4")
+
     L = layer(5, 64, 64, np.float16)
     D = G.to_dev(L)
     plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
