@@ -291,14 +291,18 @@ def main():
                         "compulsory_GBs": compulsory_bytes(L) / avg_s / 1e9,
                         "compulsory_frac": compulsory_bytes(L) / avg_s / 1e9 / PEAK_HBM_GBS}
         else:
-            ach = flops_pass / avg_s / 1e12
-            which = "dgrad" if "dgrad" in dom else ("wgrad" if "wgrad" in dom else "fwd")
+            # the backward call's single launch computes both gradients
+            parts = ("dgrad", "wgrad") if dom.startswith("bwd_fused") else \
+                (("dgrad",) if "dgrad" in dom else (("wgrad",) if "wgrad" in dom else ("fwd",)))
+            ach = len(parts) * flops_pass / avg_s / 1e12
+            flow = sum(dataflow_bytes(L, w_) for w_ in parts)
             roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_TFLOPS[arith],
                         "unit": "TFLOP/s", "frac": ach / PEAK_TFLOPS[arith], "traffic": measured_traffic(args.workload, dom),
                         "avg_kernel_ms": kernels[dom]["avg_ms"],
                         # the same launch priced as pair-list dataflow bytes against HBM
-                        "dataflow_bytes": dataflow_bytes(L, which),
-                        "dataflow_GBs": dataflow_bytes(L, which) / avg_s / 1e9}
+                        "passes_in_kernel": list(parts),
+                        "dataflow_bytes": flow,
+                        "dataflow_GBs": flow / avg_s / 1e9}
 
     line = {
         "metric": "effective TFLOP/s (2*sum|map_k|*Cin*Cout/t), %s, %s"

@@ -483,6 +483,11 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
   // fp16 tensor.  (The two gradients do not depend on each other.)
   if (n_pairs > 0 && route_of(d, p) == Route::kRows && g_policy != 1 && mfma_wgrad_supported(w)) {
     p->last_stream = d.stream;
+    // one launch for both where the shapes allow (and a small one that rounds an fp16
+    // weight gradient), else two
+    bool fused = false;
+    if ((rc = launch_fused_bwd(d, p, w, &fused))) return rc;
+    if (fused) return FGMS_OK;
     SideJob pack{}, flush{};
     const void *packed = nullptr;
     if ((rc = planned_pack_job(d, &pack, &packed))) return rc;

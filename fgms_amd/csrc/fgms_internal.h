@@ -163,6 +163,8 @@ int launch_mfma_wgrad(const WgradArgs &a);
 // Describes the weight re-layout the output-stationary kernel needs for `a` as a side job
 // (nothing is launched) and returns where the packed weights will be.
 int planned_pack_job(const GmsArgs &a, SideJob *job, const void **packed);
+// Both gradients of a layer in one launch where that is supported (*done says whether).
+int launch_fused_bwd(const GmsArgs &d, const struct Plan *p, const WgradArgs &w, bool *done);
 // Runs a side job in a launch of its own.
 int launch_side_job(const SideJob &job, hipStream_t stream);
 bool small_gms_supported(const GmsArgs &a, const Plan *p);

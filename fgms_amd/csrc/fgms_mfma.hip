@@ -32,6 +32,7 @@
 #include "fgms_device.h"
 #include "fgms_internal.h"
 #include "fgms_mma.h"
+#include "fgms_wgrad_bodies.h"
 
 namespace fgms {
 namespace {
@@ -142,6 +143,30 @@ __device__ __forceinline__ void mma_slab_raw(float16v (&acc)[2][NT], const int4v
     int4v b[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) b[nt] = raw_weight_frag<NT, S>(w_lds, s, nt, lane);
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+    }
+  }
+}
+
+// --- input-gradient weights straight from the caller's tensor --------------------------
+// The input gradient contracts over the COLUMNS of W[k] (dIn[ci] = sum over co of
+// dOut[co] * W[k][ci][co]), and those are contiguous in memory: the 8 halfs (4 floats) an
+// MFMA lane wants are one 16-byte piece of row ci.  A stage's weight tile (NT*32 rows ci x
+// 2*S chunks of the co slab) goes to LDS as it lies in memory, swizzled like a wave's
+// staging tile of gathered rows, and a fragment is one 16-byte read.  No re-layout at all.
+template <typename T, int NT, int S>
+__device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+                                              const int4v *__restrict__ w_lds, int lane) {
+  const int h = lane / 32, r = lane % 32;
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    int4v b[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[a_slot<S>(nt * 32 + r, h * S + s)];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
       const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
@@ -460,23 +485,16 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 // written to LDS after the MFMAs and one barrier closes the stage.  Weights are
 // double-buffered in LDS, each wave's row tile is single-buffered (only its own
 // wave reads it).
-// RAW: `packed` is the caller's weight tensor itself (forward, fp16: see raw_weight_frag);
-// otherwise the re-laid copy pack_weight_elements makes.
-template <typename T, int NT, int S, bool RAW>
-__global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
+// RAW = 1: `packed` is the caller's weight tensor itself, forward (fp16: see raw_weight_frag);
+// RAW = 2: the same for the input gradient (see mma_slab_rawt); RAW = 0: the re-laid copy
+// pack_weight_elements makes.
+// (block_x, block_y, block_z) of a grid (tiles, column tiles, grid_z parts of a tile).
+template <typename T, int NT, int S, int RAW>
+__device__ __forceinline__ void gms_rows_body(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
-    int c_src, int c_dst, int part_stages, SideJob side) {
-  // the leading workgroups of the grid run the side job, if there is one
-  int block_x = blockIdx.x;
-  if (side.blocks) {
-    if (block_x < side.blocks) {
-      if (blockIdx.y == 0 && blockIdx.z == 0) run_side_job(side, block_x);
-      return;
-    }
-    block_x -= side.blocks;
-  }
+    int c_src, int c_dst, int part_stages, int block_x, int block_y, int block_z, int grid_z) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
   constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
@@ -494,7 +512,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
   int *idx_all = reinterpret_cast<int *>(lds + 2 * WCH + kWaves * (kWaveRows * C));
   int *gidx = idx_all + wave * 2 * kWaveRows;
   int *didx = gidx + kWaveRows;
-  const int nt0 = blockIdx.y * NT;
+  const int nt0 = block_y * NT;
   const int4v *packed4 = reinterpret_cast<const int4v *>(packed);
   const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
 
@@ -521,18 +539,18 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     if (n_off * 4 > k_vol * 3) __builtin_amdgcn_s_setprio(3);
     else if (n_off * 2 > k_vol) __builtin_amdgcn_s_setprio(1);
   }
-  // gridDim.z > 1: a tile is shared by up to gridDim.z workgroups, each takes a run
+  // grid_z > 1: a tile is shared by up to grid_z workgroups, each takes a run
   // of the tile's offsets and adds its partial result with atomics.
   bool shared_tile = false;
-  if (gridDim.z > 1) {
+  if (grid_z > 1) {
     const int n_off = __builtin_popcountll(todo);
     const int want = (n_off * slabs + part_stages - 1) / part_stages;
-    const int parts = min((int)gridDim.z, max(want, 1));
-    if ((int)blockIdx.z >= parts) return;
+    const int parts = min(grid_z, max(want, 1));
+    if (block_z >= parts) return;
     if (parts > 1) {
       shared_tile = true;
       const int per = (n_off + parts - 1) / parts;
-      for (int i = 0; i < (int)blockIdx.z * per; ++i) todo &= todo - 1;      // offsets of earlier parts
+      for (int i = 0; i < block_z * per; ++i) todo &= todo - 1;      // offsets of earlier parts
       unsigned long long mine = 0, rest = todo;
       for (int i = 0; i < per && rest; ++i) {
         mine |= rest & (0 - rest);
@@ -557,12 +575,18 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     for (int i = 0; i < NW; ++i) {
       const int e = threadIdx.x + kThreads * i;
       if (NW * kThreads == WCH || e < WCH) {
-        if constexpr (RAW) {
+        if constexpr (RAW == 1) {
           // chunk e of the tile as it lies in memory: row e / (NT*4) of the slab's 2*S*8
           // rows of W[k], 16-byte piece e % (NT*4) of the NT*32 columns from nt0*32 on
           const int row = e / (NT * 4), c = e % (NT * 4);
           wreg[i] = *reinterpret_cast<const int4v *>(
               packed + ((size_t)k * c_src + slab * (C * E) + row) * c_dst + nt0 * 32 + c * E);
+        } else if constexpr (RAW == 2) {
+          // row e / C of the NT*32 rows of W[k] from nt0*32 on (c_dst rows of c_src
+          // elements here), 16-byte piece e % C of the slab
+          const int row = e / C, c = e % C;
+          wreg[i] = *reinterpret_cast<const int4v *>(
+              packed + ((size_t)k * c_dst + nt0 * 32 + row) * c_src + (size_t)(slab * C + c) * E);
         } else {
           const int q = e / (NT * 64), rem = e % (NT * 64);
           wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
@@ -575,9 +599,11 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     for (int i = 0; i < NW; ++i) {
       const int e = threadIdx.x + kThreads * i;
       if (NW * kThreads == WCH || e < WCH) {
-        if constexpr (RAW) {
+        if constexpr (RAW == 1) {
           const int row = e / (NT * 4), c = e % (NT * 4);
           w_lds[buf * WCH + row * (NT * 4) + (c ^ raw_swizzle<NT>(row))] = wreg[i];
+        } else if constexpr (RAW == 2) {
+          w_lds[buf * WCH + a_slot<S>(e / C, e % C)] = wreg[i];
         } else {
           w_lds[buf * WCH + e] = wreg[i];
         }
@@ -632,7 +658,8 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
         int4v b[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-          if constexpr (RAW) b[nt] = raw_weight_frag<NT, S>(wl, s, nt, lane);
+          if constexpr (RAW == 1) b[nt] = raw_weight_frag<NT, S>(wl, s, nt, lane);
+          else if constexpr (RAW == 2) b[nt] = wl[a_slot<S>(nt * 32 + r, h * S + s)];
           else b[nt] = wl[(s * NT + nt) * 64 + lane];
         }
 #pragma unroll
@@ -653,7 +680,8 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
         if (next_active) gather_issue<T, S>(v, gsel, gidx, src, c_src, nslab, lane);
       }
       if (active) {
-        if constexpr (RAW) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+        if constexpr (RAW == 1) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+        else if constexpr (RAW == 2) mma_slab_rawt<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
         else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
       }
     }
@@ -679,6 +707,25 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     else
       add_rows_lds<T, NT, S, false>(acc, dst, didx, reinterpret_cast<float *>(a_lds), c_dst, nt0 * 32, lane);
   }
+}
+
+template <typename T, int NT, int S, int RAW>
+__global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
+    const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
+    const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
+    const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
+    int c_src, int c_dst, int part_stages, SideJob side) {
+  // the leading workgroups of the grid run the side job, if there is one
+  int block_x = blockIdx.x;
+  if (side.blocks) {
+    if (block_x < side.blocks) {
+      if (blockIdx.y == 0 && blockIdx.z == 0) run_side_job(side, block_x);
+      return;
+    }
+    block_x -= side.blocks;
+  }
+  gms_rows_body<T, NT, S, RAW>(src, packed, dst, nbr, block_masks, perm, tile_order, n_dst, k_vol, c_src,
+                               c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z);
 }
 
 // ---------------------------------------------------------------------------
@@ -768,13 +815,17 @@ template <typename T, int NT, int S>
 int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
                 const unsigned long long *masks, const int32_t *perm, const int32_t *tile_order,
                 int tile_grid) {
-  // fp16 forward reads the weight tensor as it is (16-byte aligned rows of the tile);
-  // everything else gets a re-laid copy, made here unless the caller already has one.
-  // (With 128-column wave tiles the transposing reads cost more than the re-layout
-  // launch they save: 128 -> 128 over 120k voxels, 99.7 us against 93.6 + 4.4 us.)
-  constexpr bool kCanRaw = sizeof(T) == 2 && NT != 4;
-  const bool raw = kCanRaw && !a.transpose_w && !a.prepacked &&
-                   reinterpret_cast<uintptr_t>(a.w) % 16 == 0 && raw_weights_enabled();
+  // With 64-column wave tiles the input gradient and the fp16 forward pass read the weight
+  // tensor as it is (16-byte aligned rows of the tile) when the caller brings no re-laid
+  // copy; the rest gets one, made here.  Measured: 64 -> 64 over 200k voxels, input gradient
+  // 48.3 us raw against 47.3 us + a 4.4 us re-layout launch (the backward call re-lays
+  // inside its other launch for free and keeps doing so); with 128-column wave tiles raw
+  // weights lose either way (128 -> 128 over 120k voxels: forward 99.7 us against
+  // 93.6 + 4.4 us, input gradient 92.9 against 87.7 + 4.4 us).  The fp32 forward pass has no
+  // transposing LDS read to use.
+  int raw = 0;
+  if (NT != 4 && !a.prepacked && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 && raw_weights_enabled())
+    raw = a.transpose_w ? 2 : (sizeof(T) == 2 ? 1 : 0);
   const T *packed = raw ? (const T *)a.w : (const T *)a.prepacked;
   if (!packed) {
     int rc = pack_weights<T>(a, s, &packed);
@@ -782,7 +833,10 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   }
   const unsigned gx = tile_order ? (unsigned)tile_grid : (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
   if (gx == 0) return a.side.kind ? launch_side_job(a.side, a.stream) : FGMS_OK;
-  auto kern = raw ? gms_rows_kernel<T, NT, S, kCanRaw> : gms_rows_kernel<T, NT, S, false>;
+  constexpr bool kCanRaw = NT != 4;
+  auto kern = raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0>
+              : raw == 1 ? gms_rows_kernel<T, NT, S, kCanRaw && sizeof(T) == 2 ? 1 : 0>
+                         : gms_rows_kernel<T, NT, S, 0>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)s.lds_rows_bytes));
@@ -805,6 +859,83 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
     kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
         s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side);
+  }
+  FGMS_HIP_TRY(hipGetLastError());
+  return FGMS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Backward in one launch: the output-stationary input gradient (gms_rows_body, weights read
+// as they lie) and the per-wave weight gradient (wgrad_wave_body) share a grid.  The two
+// do not depend on each other, and workgroups of both kinds resident on the chip at the
+// same time finish sooner than the two launches one after the other: each launch alone
+// ends in a tail of a few long workgroups, which the other kind's workgroups now fill.
+// Measured on 64 -> 64 fp16 over 200k voxels: the two kernels on two streams running
+// freely 77 us per (input gradient, weight gradient) pair against 98 us back to back;
+// ordering two streams with events costs more than that gain, one grid costs nothing
+// (83 us + a 2 us launch that rounds the fp16 weight gradient).  The input gradient's
+// workgroups come first in the grid (its longest tiles are the longest jobs of the launch;
+// dealing the two kinds alternately or the weight gradient first measured 1-2 us slower).
+// Their count is a multiple of 8, so that a workgroup's index mod 8, its XCD, is what the
+// plan's XCD-aware orders of either kind assume.
+template <typename T, int NT, int S, int BI, int BJ>
+__global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
+    const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin,
+    const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
+    const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_in, int k_vol,
+    int c_in, int c_out, int part_stages, const T *__restrict__ in, float *__restrict__ gw32,
+    const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+    const int32_t *__restrict__ omap, SliceMap smap, int row_x, int row_y, int row_z, int wgrad_x) {
+  // grid: row_x * row_y * row_z workgroups of the input gradient (tiles, column tiles,
+  // parts of a tile), then wgrad_x * (tiles of dW[k]) of the weight gradient
+  const int rows_total = row_x * row_y * row_z;
+  if ((int)blockIdx.x < rows_total) {
+    const int bx = blockIdx.x % row_x, rest = blockIdx.x / row_x;
+    gms_rows_body<T, NT, S, 2>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
+                               part_stages, bx, rest % row_y, rest / row_y, row_z);
+  } else {
+    const int j = blockIdx.x - rows_total;
+    if constexpr (BI <= 2 && BJ <= 2)
+      wgrad_wave_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, j % wgrad_x,
+                                 j / wgrad_x);
+    else
+      wgrad_wg_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, j % wgrad_x,
+                               j / wgrad_x);
+  }
+}
+
+// FGMS_FUSED_BWD=0 keeps the backward call on its two launches (for comparison).
+bool fused_bwd_enabled() {
+  static const bool on = !(getenv("FGMS_FUSED_BWD") && atoi(getenv("FGMS_FUSED_BWD")) == 0);
+  return on;
+}
+
+template <typename T, int NT, int S, int BI, int BJ>
+int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArgs &w, const WgradGeometry &g,
+                 float *acc32) {
+  // the input gradient's grid, as launch_rows lays it out (tiles padded to a multiple of 8)
+  const unsigned tiles = p->tile_in ? (unsigned)p->tile_grid_in : (unsigned)((d.n_dst + kTileRows - 1) / kTileRows);
+  const unsigned row_x = (tiles + 7) / 8 * 8;
+  const int slabs = s.c_src / (2 * S * s.E);
+  const unsigned row_y = (unsigned)(s.c_dst / (32 * NT));
+  const int64_t slots = (int64_t)num_cus() * (NT == 4 ? 2 : 3);
+  int part_stages = 1;
+  unsigned row_z = 1;
+  if ((int64_t)tiles * row_y * 2 <= slots && d.k_vol * slabs >= 8) {
+    part_stages = (d.k_vol * slabs + 1) / 2;
+    row_z = 2;
+  }
+  size_t lds = g.lds;
+  if (lds < s.lds_rows_bytes) lds = s.lds_rows_bytes;
+  auto kern = bwd_fused_kernel<T, NT, S, BI, BJ>;
+  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  {
+    ProfileScope prof("bwd_fused_kernel", d.stream);
+    kern<<<row_x * row_y * row_z + (unsigned)(g.tiles * g.ty), kThreads, lds, d.stream>>>(
+        (const T *)d.src, (const T *)d.w, (T *)d.dst, p->nbr_in, p->mask_in, p->perm_in, p->tile_in,
+        (int)d.n_dst, d.k_vol, d.c_in, d.c_out, part_stages, (const T *)w.in, acc32, w.kpos, w.imap, w.omap,
+        g.smap, (int)row_x, (int)row_y, (int)row_z, (int)g.tiles);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -862,6 +993,46 @@ int pack_weights_any(const GmsArgs &a, int S, const void **packed) {
   int rc = pack_weights<float>(a, s, &p);
   *packed = p;
   return rc;
+}
+
+// Input gradient `d` (output-stationary, through plan `p`) and weight gradient `w` of one
+// layer in one launch where bwd_fused_kernel covers the shape; *done = false (and nothing
+// launched) where it does not.
+int launch_fused_bwd(const GmsArgs &d, const Plan *p, const WgradArgs &w, bool *done) {
+  *done = false;
+  if (!fused_bwd_enabled() || !d.transpose_w || d.prepacked || d.side.kind || w.side.kind ||
+      d.k_vol != w.k_vol || d.c_in != w.c_in || d.c_out != w.c_out || d.dtype != w.dtype || d.stream != w.stream)
+    return FGMS_OK;
+  const Shape s = shape_of(d);
+  if (!s.ok || reinterpret_cast<uintptr_t>(d.w) % 16 != 0 || !raw_weights_enabled()) return FGMS_OK;
+  WgradGeometry g;
+  if (!mfma_wgrad_supported(w) || wgrad_geometry(w, &g) != FGMS_OK) return FGMS_OK;
+  float *acc32 = nullptr;
+  int rc = wgrad_accumulator(w, &acc32);
+  if (rc != FGMS_OK) return rc;
+  bool found = false;
+  // (wave tile columns NT of the input gradient, MFMA steps per slab S) follow from c_in and
+  // c_out, and so do the block counts (BI, BJ) of the weight gradient's tile
+#define FGMS_FB(TT, NTv, Sv, BIv, BJv)                                             \
+  if (!found && s.NTR == NTv && s.S == Sv && g.bi == BIv && g.bj == BJv) {          \
+    found = true;                                                                    \
+    rc = launch_fused<TT, NTv, Sv, BIv, BJv>(d, s, p, w, g, acc32);                 \
+  }
+  if (d.dtype == FGMS_F16) {
+    FGMS_FB(__half, 1, 2, 1, 1) FGMS_FB(__half, 1, 4, 1, 2) FGMS_FB(__half, 1, 4, 1, 4)
+    FGMS_FB(__half, 2, 2, 2, 1) FGMS_FB(__half, 2, 4, 2, 2) FGMS_FB(__half, 2, 4, 2, 4)
+    FGMS_FB(__half, 2, 2, 4, 1) FGMS_FB(__half, 2, 4, 4, 2) FGMS_FB(__half, 2, 4, 4, 4)
+    FGMS_FB(__half, 4, 2, 4, 1) FGMS_FB(__half, 4, 4, 4, 2) FGMS_FB(__half, 4, 4, 4, 4)
+  } else {
+    FGMS_FB(float, 1, 4, 1, 1) FGMS_FB(float, 1, 4, 1, 2) FGMS_FB(float, 1, 4, 1, 4)
+    FGMS_FB(float, 2, 4, 2, 1) FGMS_FB(float, 2, 4, 2, 2) FGMS_FB(float, 2, 4, 2, 4)
+    FGMS_FB(float, 2, 4, 4, 1) FGMS_FB(float, 2, 4, 4, 2) FGMS_FB(float, 2, 4, 4, 4)
+  }
+#undef FGMS_FB
+  if (!found) return FGMS_OK;     // (no such kernel: the caller's two launches)
+  if (rc != FGMS_OK) return rc;
+  *done = true;
+  return wgrad_finish(w, acc32);
 }
 
 int planned_pack_job(const GmsArgs &a, SideJob *job, const void **packed) {

@@ -138,3 +138,37 @@ def test_dense_grid_built_and_convolved_on_the_device(capi, side, c, dtype, tol)
     assert torch.allclose(out[v].double(), ref, rtol=1e-2 if dtype == torch.float16 else 1e-5,
                           atol=1e-2 if dtype == torch.float16 else 1e-5)
     plan.close()
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32], ids=["fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(64, 64), (32, 64), (64, 32), (32, 32)], ids=lambda s: "%dx%d" % s)
+def test_backward_in_one_launch_full_size(capi, oracle, shape, dtype):
+    """On a launch that fills the chip fgms_bwd runs both gradients of a 32/64-channel layer
+    in ONE grid (input-gradient workgroups first, weight-gradient workgroups behind them).
+    Over the 200k-voxel cloud: that kernel is the one that ran, the input gradient equals
+    the separate fgms_dgrad call bit for bit, both gradients match the CPU oracle, and a
+    second call gives the same (the fp32 scratch of the fp16 weight gradient came back
+    empty)."""
+    rng = np.random.default_rng(77)
+    vox = clouds.cloud_indoor(clouds.rng_for(2), target=200000)
+    L = clouds.submanifold_case(vox, shape[0], shape[1], dtype, rng)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(0)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    mode = G.mode_of(L["in_feats"].dtype, False)
+    args = (L["knnz"], L["imap"], L["omap"])
+    want_gi = oracle.np_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"])
+    want_gw = oracle.np_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"])
+    gi_s, _ = G.run_bwd(capi, D, plan=plan, split=True)
+    capi.profile_reset()
+    capi.profile_enable(True)
+    for _ in range(2):
+        gi_f, gw_f = G.run_bwd(capi, D, plan=plan, split=False)
+        assert np.array_equal(gi_f, gi_s)
+        G.assert_close(gi_f, want_gi, mode, "dgrad")
+        G.assert_close(gw_f, want_gw, mode, "wgrad")
+    capi.profile_enable(False)
+    names = {n for n, _ in capi.profile_records()}
+    capi.profile_reset()
+    plan.close()
+    assert names == {"bwd_fused_kernel"}, names
