@@ -105,9 +105,9 @@ int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz,
  * fgms_bwd_cuda, backend/pybind_cuda.cpp:10): input gradient and weight
  * gradient, both accumulated into caller-zeroed buffers.  separate_mid and
  * arch80 are accepted and ignored, as in the reference.  (The reference launches
- * the input gradient first; the two do not depend on each other, and with a plan
- * this library runs the weight gradient first so that its launch can also re-lay
- * the weights for the input gradient: two launches in all.)
+ * the input gradient, then the weight gradient; the two do not depend on each
+ * other, and with a plan this library runs the workgroups of both in one launch,
+ * followed for fp16 by a small one that rounds the weight gradient's fp32 sums.)
  *   in_feats_grad[in_map[j]]  += out_feats_grad[out_map[j]] @ kernel[k]^T
  *   kernel_grad[k]            += in_feats[in_map[j]]^T (x) out_feats_grad[out_map[j]]
  */
