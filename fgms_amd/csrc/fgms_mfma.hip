@@ -868,8 +868,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
 // Backward in one launch: the output-stationary input gradient (gms_rows_body, weights read
 // as they lie) and the per-wave weight gradient (wgrad_wave_body) share a grid.  The two
 // do not depend on each other, and workgroups of both kinds resident on the chip at the
-// same time finish sooner than the two launches one after the other: each launch alone
-// ends in a tail of a few long workgroups, which the other kind's workgroups now fill.
+// same time finish sooner than the two launches one after the other.
 // Measured on 64 -> 64 fp16 over 200k voxels: the two kernels on two streams running
 // freely 77 us per (input gradient, weight gradient) pair against 98 us back to back;
 // ordering two streams with events costs more than that gain, one grid costs nothing
