@@ -116,7 +116,8 @@ struct Plan {
   int band_rows;         // output rows per band
   bool bands_ok;
   // Workgroup -> tile of 256 positions for the output-stationary kernel:
-  // workgroup b runs on XCD b % 8 and takes tile tile_out[b] (or -1: none), chosen
+  // workgroup b runs on XCD b % 8 and takes tile tile_out[b] & 0xFFFFFF (or -1: none; the
+  // bits above hold the first offset the tile uses), chosen
   // so that a tile runs on the XCD that owns the eighth of the cloud most of its
   // rows lie in (their neighbours then meet in that XCD's L2).  nullptr: tile = b.
   int32_t *tile_out, *tile_in;

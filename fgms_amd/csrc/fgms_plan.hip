@@ -139,7 +139,7 @@ __global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32
 //    three long ones competing for the same SIMDs.
 //  * Every XCD takes at most cap = ceil(tiles / 8) tiles; the lightest tiles of an
 //    overfull XCD go to the XCDs that have room.
-// order[q * 8 + xcd] = tile (pre-filled with -1).  One workgroup; which of two
+// order[q * 8 + xcd] = tile | first offset << 24 (pre-filled with -1).  One workgroup; which of two
 // equally heavy tiles comes first depends on timing, the results do not.
 __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restrict__ perm,
                                                           const unsigned long long *__restrict__ block_masks,
@@ -159,16 +159,19 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restr
   }
   if (tid == 0) spill_count = 0;
   __syncthreads();
-  auto classify = [&](int t, int &home, int &pc) {
+  // entry of tile t in the table: t in the low 24 bits, the first offset the tile uses above
+  // them (the kernel starts that offset's index load before it has seen the tile's masks)
+  auto classify = [&](int t, int &home, int &pc, int &entry) {
     const int mid = min(t * 256 + 128, n_rows - 1);
     home = (int)((long long)(perm ? perm[mid] : mid) * 8 / n_rows);
     unsigned long long m = 0;
     for (int b = 4 * t; b < min(4 * t + 4, n_blocks); ++b) m |= block_masks[b];
     pc = __builtin_popcountll(m);
+    entry = t | ((m ? __builtin_ctzll(m) : 0) << 24);
   };
   for (int t = tid; t < n_tiles; t += 1024) {
-    int home, pc;
-    classify(t, home, pc);
+    int home, pc, entry;
+    classify(t, home, pc, entry);
     atomicAdd(&hist[home][pc], 1);
   }
   __syncthreads();
@@ -188,11 +191,11 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restr
     return round * cus_per_xcd + ((round & 1) ? in_round - 1 - j : j);
   };
   for (int t = tid; t < n_tiles; t += 1024) {
-    int home, pc;
-    classify(t, home, pc);
+    int home, pc, entry;
+    classify(t, home, pc, entry);
     const int rank = hist[home][pc] + atomicAdd(&cursor[home][pc], 1);
-    if (rank < cap) order[position(rank) * 8 + home] = t;
-    else spill[atomicAdd(&spill_count, 1)] = t;
+    if (rank < cap) order[position(rank) * 8 + home] = entry;
+    else spill[atomicAdd(&spill_count, 1)] = entry;
   }
   __syncthreads();
   for (int sidx = tid; sidx < spill_count; sidx += 1024) {
