@@ -24,7 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3}
+PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3}      # dense MFMA: fp16 and bf16 alike, fp32
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
@@ -294,10 +294,14 @@ def main():
             # the backward call's single launch computes both gradients
             parts = ("dgrad", "wgrad") if dom.startswith("bwd_fused") else \
                 (("dgrad",) if "dgrad" in dom else (("wgrad",) if "wgrad" in dom else ("fwd",)))
-            ach = len(parts) * flops_pass / avg_s / 1e12
+            # fp32 tensors in tf32 mode: every product is three bf16 MFMAs (hi*hi + hi*lo + lo*hi),
+            # so the matrix pipes do three times the algorithmic flop, at the 16-bit rate
+            factor, peak = (3, PEAK_TFLOPS["f16"]) if "bf16x3" in dom else (1, PEAK_TFLOPS[arith])
+            ach = factor * len(parts) * flops_pass / avg_s / 1e12
             flow = sum(dataflow_bytes(L, w_) for w_ in parts)
-            roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_TFLOPS[arith],
-                        "unit": "TFLOP/s", "frac": ach / PEAK_TFLOPS[arith], "traffic": measured_traffic(args.workload, dom),
+            roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": peak,
+                        "unit": "TFLOP/s", "frac": ach / peak, "traffic": measured_traffic(args.workload, dom),
+                        "mfma_flop_per_algorithmic_flop": factor,
                         "avg_kernel_ms": kernels[dom]["avg_ms"],
                         # the same launch priced as pair-list dataflow bytes against HBM
                         "passes_in_kernel": list(parts),

@@ -356,7 +356,7 @@ int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz, void 
                     const int32_t *out_map, int separate_mid, int arch80, int64_t n_in,
                     int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype,
                     fgms_plan_t *plan, void *stream) {
-  (void)sum_nnz; (void)qkpos; (void)arch80;
+  (void)sum_nnz; (void)qkpos;
   int rc = check_common(in_feats, kernel, out_feats, kpos, in_map, out_map, n_in, n_out, c_in,
                         c_out, k_vol, n_pairs, dtype);
   if (rc) return rc;
@@ -364,6 +364,7 @@ int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz, void 
   hipStream_t s = (hipStream_t)stream;
   GmsArgs a = fwd_args(in_feats, kernel, out_feats, kpos, in_map, out_map, n_in, n_out, c_in,
                        c_out, k_vol, n_pairs, dtype, s);
+  a.reduced = arch80 != 0 && dtype == FGMS_F32;
   if (separate_mid) {
     // centre product first and overwriting, as the beta = 0 GEMM of the reference
     const size_t esz = dtype == FGMS_F16 ? 2 : 4;
@@ -382,7 +383,7 @@ int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_fe
              const int32_t *out_map, int separate_mid, int arch80, int64_t n_in, int64_t n_out,
              int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype, fgms_plan_t *plan,
              void *stream) {
-  (void)sum_nnz; (void)arch80;
+  (void)sum_nnz;
   int rc = check_common(in_feats, kernel, out_feats, kernel_pos, in_map, out_map, n_in, n_out,
                         c_in, c_out, k_vol, n_pairs, dtype);
   if (rc) return rc;
@@ -409,6 +410,7 @@ int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_fe
   hipStream_t s = (hipStream_t)stream;
   GmsArgs a = fwd_args(in_feats, kernel, out_feats, kernel_pos, in_map, out_map, n_in, n_out,
                        c_in, c_out, k_vol, total, dtype, s);
+  a.reduced = arch80 != 0 && dtype == FGMS_F32;
   if ((rc = run_gms(a, (const Plan *)plan))) return rc;
   if (separate_mid) {
     GmsArgs d = a;

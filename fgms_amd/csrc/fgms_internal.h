@@ -62,6 +62,9 @@ struct GmsArgs {
   int64_t n_dense;
   int dtype;
   hipStream_t stream;
+  // fp32 tensors in the reference's "tf32" mode: products may be rounded to tf32 precision
+  // (10 mantissa bits) or better, sums stay fp32
+  bool reduced;
   const void *prepacked;   // output-stationary kernel only: the weights are already re-laid here
   SideJob side;            // ... and this rides along with its launch
 };

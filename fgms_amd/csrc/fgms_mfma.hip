@@ -176,6 +176,117 @@ __device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[2][NT], const int4
   }
 }
 
+// --- fp32 tensors, products in split bf16 ("tf32" mode) ------------------------------------
+// gfx950 has no tf32 matrix instruction, and its fp32 one runs at a sixteenth of the 16-bit
+// rate.  Where the caller allows tf32 precision for the products (10 mantissa bits), every
+// fp32 value is split into two bf16 numbers, x = hi + lo + O(2^-17 x), and a product becomes
+// three bf16 MFMAs into the fp32 accumulator: hi*hi + hi*lo + lo*hi.  The dropped lo*lo term
+// is below 2^-16 of the product, so this is more exact than tf32, at 3/16 of the fp32 matrix
+// time.  Rows are split when they go from registers to LDS, the weights by their re-layout
+// kernel.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef int int2v __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void split_bf16(float x, __bf16 &hi, __bf16 &lo) {
+  hi = (__bf16)x;
+  const float h = (float)hi;
+  // (an infinite or NaN value stays in hi alone)
+  lo = (__bf16)(__builtin_fabsf(h) < __builtin_inff() ? x - h : 0.f);
+}
+
+// Slot (16 bytes = 8 bf16) of a wave's split staging tile: row-major, a row holds its 32
+// values of the slab as 4 chunks of hi followed by 4 chunks of lo (128 bytes, as the fp32
+// row did); the XOR spreads the 8 rows one b128 read pass touches over all banks.
+__device__ __forceinline__ int a_bf_slot(int row, int part, int j) {
+  return row * 8 + part * 4 + (j ^ ((row >> 1) & 3));
+}
+
+// registers -> LDS for the split tile: lane pairs hold the two fp32 chunks that make one
+// bf16 chunk; the even lane ends up with the 8 hi values, the odd one with the 8 lo values.
+__device__ __forceinline__ void gather_commit_bf3(int4v *__restrict__ a_lds, int4v (&v)[8],
+                                                  const int (&g)[8], int lane) {
+  const bool odd = lane & 1;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int slot = it * 64 + lane;
+    const int row = slot / 8, c = slot % 8;
+    const float4v x = g[it] < 0 ? float4v{0.f, 0.f, 0.f, 0.f} : __builtin_bit_cast(float4v, v[it]);
+    bf16x4 hi, lo;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __bf16 h, l;
+      split_bf16(x[i], h, l);
+      hi[i] = h;
+      lo[i] = l;
+    }
+    const int2v h2 = __builtin_bit_cast(int2v, hi), l2 = __builtin_bit_cast(int2v, lo);
+    // the even lane hands over its lo half and takes the odd lane's hi half
+    const int got0 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[0] : l2[0])));
+    const int got1 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[1] : l2[1])));
+    const int4v out = odd ? int4v{got0, got1, l2[0], l2[1]} : int4v{h2[0], h2[1], got0, got1};
+    a_lds[a_bf_slot(row, odd ? 1 : 0, c / 2)] = out;
+  }
+}
+
+// acc[mt][nt] += A(slab) x W(slab), both split; weights in LDS as [k-step][nt][hi, lo][lane].
+template <int NT>
+__device__ __forceinline__ void mma_slab_bf3(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+                                             const int4v *__restrict__ w_lds, int lane) {
+  const int h = lane / 32, r = lane % 32;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    bf16x8 bh[NT], bl[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      bh[nt] = __builtin_bit_cast(bf16x8, w_lds[((s * NT + nt) * 2 + 0) * 64 + lane]);
+      bl[nt] = __builtin_bit_cast(bf16x8, w_lds[((s * NT + nt) * 2 + 1) * 64 + lane]);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const bf16x8 ah = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 0, s * 2 + h)]);
+      const bf16x8 al = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 1, s * 2 + h)]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[nt], acc[mt][nt], 0, 0, 0);
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[nt], acc[mt][nt], 0, 0, 0);
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[nt], acc[mt][nt], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// Split weights in the order mma_slab_bf3 reads them: chunk
+//   ((((k * slabs + slab) * 2 + s) * nts + nt) * 2 + part) * 64 + lane
+// holds the 8 values W[k][slab*32 + s*16 + (lane/32)*8 + 0..7][nt*32 + lane%32], hi (part 0)
+// or lo (part 1).  One thread per chunk pair.
+__global__ void pack_weights_bf3_kernel(const float *__restrict__ w, int4v *__restrict__ packed,
+                                        int k_vol, int c_in, int c_out) {
+  const int slabs = c_in / 32, nts = c_out / 32;
+  const size_t total = (size_t)k_vol * slabs * 2 * nts * 64;
+  for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
+       t += (size_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(t % 64);
+    size_t q = t / 64;
+    const int nt = (int)(q % nts); q /= nts;
+    const int s = (int)(q % 2); q /= 2;
+    const int slab = (int)(q % slabs);
+    const int k = (int)(q / slabs);
+    const int cs0 = slab * 32 + s * 16 + (lane / 32) * 8, cd = nt * 32 + lane % 32;
+    bf16x8 hi, lo;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      __bf16 h, l;
+      split_bf16(w[((size_t)k * c_in + cs0 + e) * c_out + cd], h, l);
+      hi[e] = h;
+      lo[e] = l;
+    }
+    const size_t base = (t / 64) * 128 + lane;
+    packed[base] = __builtin_bit_cast(int4v, hi);
+    packed[base + 64] = __builtin_bit_cast(int4v, lo);
+  }
+}
+
 // Writes a wave's accumulators.  Accumulator register r of lane l holds row
 // (r / 4) * 8 + (l / 32) * 4 + r % 4 and column l % 32 of its 32x32 tile.  For
 // fp16 two lanes swap one value each so that every lane owns two neighbouring
@@ -507,8 +618,9 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 // double-buffered in LDS, each wave's row tile is single-buffered (only its own
 // wave reads it).
 // RAW = 1: `packed` is the caller's weight tensor itself, forward (fp16: see raw_weight_frag);
-// RAW = 2: the same for the input gradient (see mma_slab_rawt); RAW = 0: the re-laid copy
-// pack_weight_elements makes.
+// RAW = 2: the same for the input gradient (see mma_slab_rawt); RAW = 3: fp32 tensors with
+// products in split bf16 (see mma_slab_bf3), `packed` from pack_weights_bf3_kernel; RAW = 0:
+// the re-laid copy pack_weight_elements makes.
 // (block_x, block_y, block_z) of a grid (tiles, column tiles, grid_z parts of a tile).
 template <typename T, int NT, int S, int RAW>
 __device__ __forceinline__ void gms_rows_body(
@@ -524,7 +636,7 @@ __device__ __forceinline__ void gms_rows_body(
   __shared__ unsigned long long wg_mask;
   // fp32 only: its MFMA phase is long enough (4 k clocks a stage) to absorb the loads'
   // issue waits; for fp16 the interleaved stage measured 2 us slower per launch
-  constexpr bool kInterleave = sizeof(T) == 4;
+  constexpr bool kInterleave = sizeof(T) == 4 && RAW != 3;
   const int slabs = c_src / (C * E);
   const int nts = c_dst / 32;
   int4v *w_lds = lds;                                     // [2][WCH]
@@ -619,6 +731,10 @@ __device__ __forceinline__ void gms_rows_body(
           const int row = e / C, c = e % C;
           wreg[i] = *reinterpret_cast<const int4v *>(
               packed + ((size_t)k * c_dst + nt0 * 32 + row) * c_src + (size_t)(slab * C + c) * E);
+        } else if constexpr (RAW == 3) {
+          // k-step e / (NT*128) of the stage, then [nt][hi, lo][lane]
+          const int q = e / (NT * 128), rem = e % (NT * 128);
+          wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * 2 + q) * nts + nt0) * 128 + rem];
         } else {
           const int q = e / (NT * 64), rem = e % (NT * 64);
           wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
@@ -660,7 +776,7 @@ __device__ __forceinline__ void gms_rows_body(
   weights_issue(wreg, k, 0);
   if (active) gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
   weights_commit(wreg, 0);
-  if (active) gather_commit<S>(a_lds, v, gsel, lane);
+  if (active) { if constexpr (RAW == 3) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
   __syncthreads();
 
   int buf = 0;
@@ -714,12 +830,13 @@ __device__ __forceinline__ void gms_rows_body(
       if (active) {
         if constexpr (RAW == 1) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
         else if constexpr (RAW == 2) mma_slab_rawt<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+        else if constexpr (RAW == 3) mma_slab_bf3<NT>(acc, a_lds, w_lds + buf * WCH, lane);
         else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
       }
     }
     if (!has_next) break;
     wave_lds_fence();
-    if (next_active) gather_commit<S>(a_lds, v, gsel, lane);
+    if (next_active) { if constexpr (RAW == 3) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
     weights_commit(wreg, buf ^ 1);
     if (nk != k) {
       k_nxt = todo ? __builtin_ctzll(todo) : -1;
@@ -837,6 +954,12 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   return FGMS_OK;
 }
 
+// FGMS_SPLIT_BF16=0 keeps fp32 tensors on fp32 MFMAs in "tf32" mode too (for comparison).
+bool split_bf16_enabled() {
+  static const bool on = !(getenv("FGMS_SPLIT_BF16") && atoi(getenv("FGMS_SPLIT_BF16")) == 0);
+  return on;
+}
+
 // FGMS_RAW_WEIGHTS=0 keeps the forward pass on re-laid weights (for comparison).
 bool raw_weights_enabled() {
   static const bool on = !(getenv("FGMS_RAW_WEIGHTS") && atoi(getenv("FGMS_RAW_WEIGHTS")) == 0);
@@ -858,15 +981,31 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   int raw = 0;
   if (NT != 4 && !a.prepacked && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 && raw_weights_enabled())
     raw = a.transpose_w ? 2 : (sizeof(T) == 2 ? 1 : 0);
+  // fp32 forward in "tf32" mode: products in split bf16 (three 16-bit MFMAs instead of
+  // sixteen fp32 ones per product tile); needs whole 32-channel slabs
+  constexpr bool kCanSplit = sizeof(T) == 4 && S == 4 && NT != 4;
+  const bool split = kCanSplit && a.reduced && !a.transpose_w && !a.prepacked && split_bf16_enabled();
   const T *packed = raw ? (const T *)a.w : (const T *)a.prepacked;
-  if (!packed) {
+  if (split) {
+    void *ws = nullptr;
+    const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+    int rc = workspace_get(a.stream, 0, n * sizeof(float), &ws);
+    if (rc != FGMS_OK) return rc;
+    size_t blocks = (n / 8 + 255) / 256;
+    pack_weights_bf3_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, a.stream>>>(
+        (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out);
+    FGMS_HIP_TRY(hipGetLastError());
+    packed = (const T *)ws;
+    raw = 3;
+  } else if (!packed) {
     int rc = pack_weights<T>(a, s, &packed);
     if (rc != FGMS_OK) return rc;
   }
   const unsigned gx = tile_order ? (unsigned)tile_grid : (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
   if (gx == 0) return a.side.kind ? launch_side_job(a.side, a.stream) : FGMS_OK;
   constexpr bool kCanRaw = NT != 4;
-  auto kern = raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0>
+  auto kern = raw == 3   ? gms_rows_kernel<T, NT, S, kCanSplit ? 3 : 0>
+              : raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0>
               : raw == 1 ? gms_rows_kernel<T, NT, S, kCanRaw && sizeof(T) == 2 ? 1 : 0>
                          : gms_rows_kernel<T, NT, S, 0>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -887,7 +1026,9 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
     gz = 2;
   }
   {
-    ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)", a.stream);
+    ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : raw == 3 ? "gms_rows_kernel(fwd, bf16x3)"
+                                                                          : "gms_rows_kernel(fwd)",
+                      a.stream);
     kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
         s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side);

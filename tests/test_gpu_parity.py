@@ -370,3 +370,39 @@ def test_result_rows_not_16_byte_aligned(capi, oracle, dtype):
     ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
     G.assert_close(out.cpu().numpy(), ref, G.mode_of(dtype), "fwd into an unaligned result")
     assert not buf[:2].any() and not buf[2 + D["n_out"] * 64:].any()
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (32, 64), (96, 32)], ids=lambda s: "%dx%d" % s)
+def test_tf32_mode_multiplies_in_split_bf16(capi, oracle, shape):
+    """fp32 tensors with arch80 set (the reference's tf32 mode): the output-stationary
+    forward kernel splits every value into two bf16 numbers and multiplies with three
+    16-bit MFMAs.  That path is the one that runs, and it is far inside the mode's
+    tolerance: at most 1e-4 of the result's rms where tf32 itself would be allowed 1e-2
+    (measured 5e-6).  Non-finite inputs stay non-finite only where they are used."""
+    L = layer(19, shape[0], shape[1], np.float32)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(4)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
+    capi.profile_reset()
+    capi.profile_enable(True)
+    for fused in (True, False):
+        out = G.run_fwd(capi, D, fused=fused, arch80=True, plan=plan)
+        G.assert_close(out, ref, "tf32", "tf32-mode forward")
+        rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+        assert np.abs(out - ref).max() <= 1e-4 * rms
+    capi.profile_enable(False)
+    names = {n for n, _ in capi.profile_records()}
+    capi.profile_reset()
+    assert names == {"gms_rows_kernel(fwd, bf16x3)"}, names
+    # an infinite input value reaches exactly the output rows that use its row
+    D2 = dict(D)
+    x = D["in_feats"].clone()
+    x[5, 3] = float("inf")
+    D2["in_feats"] = x
+    out = G.run_fwd(capi, D2, fused=True, arch80=True, plan=plan)
+    users = np.unique(L["omap"][L["imap"] == 5])
+    bad = np.where(~np.isfinite(out).all(axis=1))[0]
+    assert set(bad) == set(users)
+    plan.close()
+    capi.set_kernel_policy(0)
