@@ -21,8 +21,12 @@
  *   - dtype: FGMS_F32 or FGMS_F16 for features, weights and gradients alike
  *     (the reference keys on in_feats.scalar_type(), backend/spconv.cu:47-48).
  *   - arch80: for FGMS_F32, non-zero = "tf32 mode" in the reference
- *     (backend/spconv.cu:67-68,213).  gfx950 has no xf32 MFMA: both modes run
- *     the fp32 MFMA kernels, so tf32 mode is simply more exact than asked.
+ *     (backend/spconv.cu:67-68,213): the products may be rounded to tf32
+ *     precision, the sums are fp32.  gfx950 has no tf32 matrix instruction;
+ *     the forward pass with a plan then multiplies in split bf16 (every value
+ *     as hi + lo, three 16-bit MFMAs per product: about 2^-16 relative error,
+ *     finer than tf32, at twice the speed of the fp32 kernels).  Everything
+ *     else, and arch80 = 0, runs the fp32 MFMA kernels.
  *   - stream: a hipStream_t (NULL = the null stream).  All work is enqueued on
  *     it; calls return without waiting for the GPU, as the reference's do.
  *   - plan: optional (NULL allowed) handle from fgms_plan_create for the same

@@ -35,7 +35,10 @@ for shape, dtype in (((64, 64), np.float16), ((128, 128), np.float16), ((32, 64)
         gi, gw = G.run_bwd(capi, D, plan=plan)
         G.assert_close(gi, oracle.np_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"]), mode, "dgrad")
         G.assert_close(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"]), mode, "wgrad")
-    G.assert_close(out, oracle.np_fwd(L["in_feats"], L["kernel"], *args, L["n_out"]), mode, "fwd")
+    want = oracle.np_fwd(L["in_feats"], L["kernel"], *args, L["n_out"])
+    G.assert_close(out, want, mode, "fwd")
+    if dtype == np.float32:
+        G.assert_close(G.run_fwd(capi, D, fused=True, arch80=True, plan=plan), want, "tf32", "tf32-mode fwd")
     capi.profile_enable(False)
     names |= {n for n, _ in capi.profile_records()}
     plan.close()
@@ -56,6 +59,13 @@ def run_child(env_extra):
 def test_default_settings_run_the_backward_in_one_grid():
     names = run_child({})
     assert "bwd_fused_kernel" in names and "wgrad_wave_kernel" not in names, names
+    assert "gms_rows_kernel(fwd, bf16x3)" in names, names
+
+
+def test_tf32_mode_on_fp32_matrix_instructions():
+    """FGMS_SPLIT_BF16=0: fp32 tensors in tf32 mode run the fp32 kernels."""
+    names = run_child({"FGMS_SPLIT_BF16": "0"})
+    assert "gms_rows_kernel(fwd, bf16x3)" not in names and "gms_rows_kernel(fwd)" in names, names
 
 
 def test_backward_on_two_launches():
