@@ -1178,7 +1178,7 @@ int launch_fused_bwd(const GmsArgs &d, const Plan *p, const WgradArgs &w, bool *
   const Shape s = shape_of(d);
   if (!s.ok || reinterpret_cast<uintptr_t>(d.w) % 16 != 0 || !raw_weights_enabled()) return FGMS_OK;
   WgradGeometry g;
-  if (!mfma_wgrad_supported(w) || wgrad_geometry(w, &g) != FGMS_OK) return FGMS_OK;
+  if (!mfma_wgrad_supported(w) || wgrad_geometry(w, &g, true) != FGMS_OK) return FGMS_OK;
   float *acc32 = nullptr;
   int rc = wgrad_accumulator(w, &acc32);
   if (rc != FGMS_OK) return rc;

@@ -463,7 +463,8 @@ struct WgradGeometry {
   bool wave;       // wgrad_wave_body, else wgrad_wg_body
   size_t lds;      // dynamic LDS
 };
-int wgrad_geometry(const WgradArgs &a, WgradGeometry *g);
+// shares_grid: the launch also holds the input gradient's workgroups.
+int wgrad_geometry(const WgradArgs &a, WgradGeometry *g, bool shares_grid = false);
 // Where the kernels accumulate: the caller's fp32 tensor, or for fp16 the stream's fp32
 // scratch (zero between calls), which wgrad_finish rounds into the caller's tensor and
 // clears again in a launch of its own.
