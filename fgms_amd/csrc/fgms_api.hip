@@ -459,7 +459,7 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
              const int32_t *in_map, const int32_t *out_map, int separate_mid, int arch80,
              int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs,
              int dtype, fgms_plan_t *plan, void *stream) {
-  (void)sum_nnz; (void)qkpos; (void)separate_mid; (void)arch80;
+  (void)sum_nnz; (void)qkpos; (void)separate_mid;
   int rc = check_common(out_feats_grad, kernel, in_feats_grad, kpos, in_map, out_map, n_in, n_out,
                         c_in, c_out, k_vol, n_pairs, dtype);
   if (rc) return rc;
@@ -473,12 +473,14 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
   d.n_src = n_out; d.n_dst = n_in; d.c_in = c_in; d.c_out = c_out; d.k_vol = k_vol;
   d.n_pairs = n_pairs; d.transpose_w = true; d.dense_k = -1; d.n_dense = 0; d.dtype = dtype;
   d.stream = (hipStream_t)stream;
+  d.reduced = arch80 != 0 && dtype == FGMS_F32;     // (the reference's backward is tf32 whenever the tensors are fp32)
   WgradArgs w{};
   w.in = in_feats; w.gout = out_feats_grad; w.gw = kernel_grad; w.kpos = kpos;
   w.imap = in_map; w.omap = out_map; w.n_in = n_in; w.n_out = n_out; w.c_in = c_in;
   w.c_out = c_out; w.k_vol = k_vol; w.n_pairs = n_pairs; w.dtype = dtype;
   w.stream = (hipStream_t)stream;
   w.plan = p;
+  w.reduced = d.reduced;
   // Both gradients through their main kernels: two launches instead of four.  The weight
   // gradient goes first and its launch also re-lays the weights for the input gradient,
   // whose launch in turn also rounds the weight gradient's fp32 sums into the caller's

@@ -82,6 +82,7 @@ struct WgradArgs {
   int dtype;
   hipStream_t stream;
   const struct Plan *plan;   // optional
+  bool reduced;              // fp32 tensors: products may be rounded to tf32 precision or better
   SideJob side;              // MFMA kernels only: rides along with the launch
   // MFMA kernels, fp16: do not launch the fp32 -> fp16 flush of the accumulator; describe
   // it in *deferred_flush instead, for the caller to attach to its next launch
@@ -171,6 +172,7 @@ int planned_pack_job(const GmsArgs &a, SideJob *job, const void **packed);
 int launch_fused_bwd(const GmsArgs &d, const struct Plan *p, const WgradArgs &w, bool *done);
 // Runs a side job in a launch of its own.
 int launch_side_job(const SideJob &job, hipStream_t stream);
+bool split_bf16_enabled();   // products of fp32 tensors in split bf16 where the caller allows tf32 precision
 bool small_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_small_gms(const GmsArgs &a, const Plan *p);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);

@@ -184,17 +184,6 @@ __device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[2][NT], const int4
 // is below 2^-16 of the product, so this is more exact than tf32, at 3/16 of the fp32 matrix
 // time.  Rows are split when they go from registers to LDS, the weights by their re-layout
 // kernel.
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef int int2v __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ void split_bf16(float x, __bf16 &hi, __bf16 &lo) {
-  hi = (__bf16)x;
-  const float h = (float)hi;
-  // (an infinite or NaN value stays in hi alone)
-  lo = (__bf16)(__builtin_fabsf(h) < __builtin_inff() ? x - h : 0.f);
-}
-
 // Slot (16 bytes = 8 bf16) of a wave's split staging tile: row-major, a row holds its 32
 // values of the slab as 4 chunks of hi followed by 4 chunks of lo (128 bytes, as the fp32
 // row did); the XOR spreads the 8 rows one b128 read pass touches over all banks.
@@ -202,30 +191,36 @@ __device__ __forceinline__ int a_bf_slot(int row, int part, int j) {
   return row * 8 + part * 4 + (j ^ ((row >> 1) & 3));
 }
 
-// registers -> LDS for the split tile: lane pairs hold the two fp32 chunks that make one
-// bf16 chunk; the even lane ends up with the 8 hi values, the odd one with the 8 lo values.
+// One fp32 chunk (4 values; chunk c of its row's slab) split and written to a split tile.
+// Lane pairs hold the two fp32 chunks that make one bf16 chunk; they exchange halves, so the
+// even lane ends up with the 8 hi values and the odd one with the 8 lo values and each
+// still writes one 16-byte chunk.
+__device__ __forceinline__ void split_and_store(int4v *__restrict__ tile, const float4v &x, int row, int c,
+                                                int lane) {
+  const bool odd = lane & 1;
+  bf16x4 hi, lo;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    __bf16 h, l;
+    split_bf16(x[i], h, l);
+    hi[i] = h;
+    lo[i] = l;
+  }
+  const int2v h2 = __builtin_bit_cast(int2v, hi), l2 = __builtin_bit_cast(int2v, lo);
+  // the even lane hands over its lo half and takes the odd lane's hi half
+  const int got0 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[0] : l2[0])));
+  const int got1 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[1] : l2[1])));
+  tile[a_bf_slot(row, odd ? 1 : 0, c / 2)] = odd ? int4v{got0, got1, l2[0], l2[1]} : int4v{h2[0], h2[1], got0, got1};
+}
+
+// registers -> LDS for the split tile of gathered rows (absent rows as zeros).
 __device__ __forceinline__ void gather_commit_bf3(int4v *__restrict__ a_lds, int4v (&v)[8],
                                                   const int (&g)[8], int lane) {
-  const bool odd = lane & 1;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int slot = it * 64 + lane;
-    const int row = slot / 8, c = slot % 8;
     const float4v x = g[it] < 0 ? float4v{0.f, 0.f, 0.f, 0.f} : __builtin_bit_cast(float4v, v[it]);
-    bf16x4 hi, lo;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      __bf16 h, l;
-      split_bf16(x[i], h, l);
-      hi[i] = h;
-      lo[i] = l;
-    }
-    const int2v h2 = __builtin_bit_cast(int2v, hi), l2 = __builtin_bit_cast(int2v, lo);
-    // the even lane hands over its lo half and takes the odd lane's hi half
-    const int got0 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[0] : l2[0])));
-    const int got1 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[1] : l2[1])));
-    const int4v out = odd ? int4v{got0, got1, l2[0], l2[1]} : int4v{h2[0], h2[1], got0, got1};
-    a_lds[a_bf_slot(row, odd ? 1 : 0, c / 2)] = out;
+    split_and_store(a_lds, x, slot / 8, slot % 8, lane);
   }
 }
 
@@ -241,6 +236,34 @@ __device__ __forceinline__ void mma_slab_bf3(float16v (&acc)[2][NT], const int4v
     for (int nt = 0; nt < NT; ++nt) {
       bh[nt] = __builtin_bit_cast(bf16x8, w_lds[((s * NT + nt) * 2 + 0) * 64 + lane]);
       bl[nt] = __builtin_bit_cast(bf16x8, w_lds[((s * NT + nt) * 2 + 1) * 64 + lane]);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const bf16x8 ah = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 0, s * 2 + h)]);
+      const bf16x8 al = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 1, s * 2 + h)]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[nt], acc[mt][nt], 0, 0, 0);
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[nt], acc[mt][nt], 0, 0, 0);
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[nt], acc[mt][nt], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// The same for the input gradient: the weight tile (NT*32 rows of W[k], the slab's 32 columns)
+// was split on its way to LDS like a tile of gathered rows (RAW = 4).
+template <int NT>
+__device__ __forceinline__ void mma_slab_bf3t(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+                                              const int4v *__restrict__ w_lds, int lane) {
+  const int h = lane / 32, r = lane % 32;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    bf16x8 bh[NT], bl[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      bh[nt] = __builtin_bit_cast(bf16x8, w_lds[a_bf_slot(nt * 32 + r, 0, s * 2 + h)]);
+      bl[nt] = __builtin_bit_cast(bf16x8, w_lds[a_bf_slot(nt * 32 + r, 1, s * 2 + h)]);
     }
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
@@ -619,8 +642,9 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 // wave reads it).
 // RAW = 1: `packed` is the caller's weight tensor itself, forward (fp16: see raw_weight_frag);
 // RAW = 2: the same for the input gradient (see mma_slab_rawt); RAW = 3: fp32 tensors with
-// products in split bf16 (see mma_slab_bf3), `packed` from pack_weights_bf3_kernel; RAW = 0:
-// the re-laid copy pack_weight_elements makes.
+// products in split bf16 (see mma_slab_bf3), `packed` from pack_weights_bf3_kernel; RAW = 4:
+// the input gradient in split bf16, weights read as they lie and split on their way to LDS;
+// RAW = 0: the re-laid copy pack_weight_elements makes.
 // (block_x, block_y, block_z) of a grid (tiles, column tiles, grid_z parts of a tile).
 template <typename T, int NT, int S, int RAW>
 __device__ __forceinline__ void gms_rows_body(
@@ -636,7 +660,7 @@ __device__ __forceinline__ void gms_rows_body(
   __shared__ unsigned long long wg_mask;
   // fp32 only: its MFMA phase is long enough (4 k clocks a stage) to absorb the loads'
   // issue waits; for fp16 the interleaved stage measured 2 us slower per launch
-  constexpr bool kInterleave = sizeof(T) == 4 && RAW != 3;
+  constexpr bool kInterleave = sizeof(T) == 4 && RAW != 3 && RAW != 4;
   const int slabs = c_src / (C * E);
   const int nts = c_dst / 32;
   int4v *w_lds = lds;                                     // [2][WCH]
@@ -725,7 +749,7 @@ __device__ __forceinline__ void gms_rows_body(
           const int row = e / (NT * 4), c = e % (NT * 4);
           wreg[i] = *reinterpret_cast<const int4v *>(
               packed + ((size_t)k * c_src + slab * (C * E) + row) * c_dst + nt0 * 32 + c * E);
-        } else if constexpr (RAW == 2) {
+        } else if constexpr (RAW == 2 || RAW == 4) {
           // row e / C of the NT*32 rows of W[k] from nt0*32 on (c_dst rows of c_src
           // elements here), 16-byte piece e % C of the slab
           const int row = e / C, c = e % C;
@@ -752,6 +776,8 @@ __device__ __forceinline__ void gms_rows_body(
           w_lds[buf * WCH + row * (NT * 4) + (c ^ raw_swizzle<NT>(row))] = wreg[i];
         } else if constexpr (RAW == 2) {
           w_lds[buf * WCH + a_slot<S>(e / C, e % C)] = wreg[i];
+        } else if constexpr (RAW == 4) {
+          split_and_store(w_lds + buf * WCH, __builtin_bit_cast(float4v, wreg[i]), e / C, e % C, lane);
         } else {
           w_lds[buf * WCH + e] = wreg[i];
         }
@@ -776,7 +802,7 @@ __device__ __forceinline__ void gms_rows_body(
   weights_issue(wreg, k, 0);
   if (active) gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
   weights_commit(wreg, 0);
-  if (active) { if constexpr (RAW == 3) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
+  if (active) { if constexpr (RAW == 3 || RAW == 4) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
   __syncthreads();
 
   int buf = 0;
@@ -831,12 +857,13 @@ __device__ __forceinline__ void gms_rows_body(
         if constexpr (RAW == 1) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
         else if constexpr (RAW == 2) mma_slab_rawt<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
         else if constexpr (RAW == 3) mma_slab_bf3<NT>(acc, a_lds, w_lds + buf * WCH, lane);
+        else if constexpr (RAW == 4) mma_slab_bf3t<NT>(acc, a_lds, w_lds + buf * WCH, lane);
         else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
       }
     }
     if (!has_next) break;
     wave_lds_fence();
-    if (next_active) { if constexpr (RAW == 3) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
+    if (next_active) { if constexpr (RAW == 3 || RAW == 4) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
     weights_commit(wreg, buf ^ 1);
     if (nk != k) {
       k_nxt = todo ? __builtin_ctzll(todo) : -1;
@@ -954,12 +981,6 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   return FGMS_OK;
 }
 
-// FGMS_SPLIT_BF16=0 keeps fp32 tensors on fp32 MFMAs in "tf32" mode too (for comparison).
-bool split_bf16_enabled() {
-  static const bool on = !(getenv("FGMS_SPLIT_BF16") && atoi(getenv("FGMS_SPLIT_BF16")) == 0);
-  return on;
-}
-
 // FGMS_RAW_WEIGHTS=0 keeps the forward pass on re-laid weights (for comparison).
 bool raw_weights_enabled() {
   static const bool on = !(getenv("FGMS_RAW_WEIGHTS") && atoi(getenv("FGMS_RAW_WEIGHTS")) == 0);
@@ -985,6 +1006,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   // sixteen fp32 ones per product tile); needs whole 32-channel slabs
   constexpr bool kCanSplit = sizeof(T) == 4 && S == 4 && NT != 4;
   const bool split = kCanSplit && a.reduced && !a.transpose_w && !a.prepacked && split_bf16_enabled();
+  if (kCanSplit && a.reduced && raw == 2 && split_bf16_enabled()) raw = 4;   // (the input gradient splits as it reads)
   const T *packed = raw ? (const T *)a.w : (const T *)a.prepacked;
   if (split) {
     void *ws = nullptr;
@@ -1004,7 +1026,8 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   const unsigned gx = tile_order ? (unsigned)tile_grid : (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
   if (gx == 0) return a.side.kind ? launch_side_job(a.side, a.stream) : FGMS_OK;
   constexpr bool kCanRaw = NT != 4;
-  auto kern = raw == 3   ? gms_rows_kernel<T, NT, S, kCanSplit ? 3 : 0>
+  auto kern = raw == 4   ? gms_rows_kernel<T, NT, S, kCanSplit ? 4 : 0>
+              : raw == 3 ? gms_rows_kernel<T, NT, S, kCanSplit ? 3 : 0>
               : raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0>
               : raw == 1 ? gms_rows_kernel<T, NT, S, kCanRaw && sizeof(T) == 2 ? 1 : 0>
                          : gms_rows_kernel<T, NT, S, 0>;
@@ -1026,8 +1049,9 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
     gz = 2;
   }
   {
-    ProfileScope prof(a.transpose_w ? "gms_rows_kernel(dgrad)" : raw == 3 ? "gms_rows_kernel(fwd, bf16x3)"
-                                                                          : "gms_rows_kernel(fwd)",
+    ProfileScope prof(raw == 4   ? "gms_rows_kernel(dgrad, bf16x3)"
+                      : raw == 3 ? "gms_rows_kernel(fwd, bf16x3)"
+                      : a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)",
                       a.stream);
     kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
@@ -1050,7 +1074,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
 // dealing the two kinds alternately or the weight gradient first measured 1-2 us slower).
 // Their count is a multiple of 8, so that a workgroup's index mod 8, its XCD, is what the
 // plan's XCD-aware orders of either kind assume.
-template <typename T, int NT, int S, int BI, int BJ>
+template <typename T, int NT, int S, int BI, int BJ, int RAWD>
 __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
     const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
@@ -1063,13 +1087,13 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
   const int rows_total = row_x * row_y * row_z;
   if ((int)blockIdx.x < rows_total) {
     const int bx = blockIdx.x % row_x, rest = blockIdx.x / row_x;
-    gms_rows_body<T, NT, S, 2>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
+    gms_rows_body<T, NT, S, RAWD>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
                                part_stages, bx, rest % row_y, rest / row_y, row_z);
   } else {
     const int j = blockIdx.x - rows_total;
     if constexpr (BI <= 2 && BJ <= 2)
-      wgrad_wave_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, j % wgrad_x,
-                                 j / wgrad_x);
+      wgrad_wave_body<T, BI, BJ, RAWD == 4>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap,
+                                            j % wgrad_x, j / wgrad_x);
     else
       wgrad_wg_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, j % wgrad_x,
                                j / wgrad_x);
@@ -1099,7 +1123,11 @@ int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArg
   }
   size_t lds = g.lds;
   if (lds < s.lds_rows_bytes) lds = s.lds_rows_bytes;
-  auto kern = bwd_fused_kernel<T, NT, S, BI, BJ>;
+  // RAWD: how the input gradient reads the weights (2: as they lie; 4: also split into bf16
+  // pairs, for fp32 tensors whose caller allows tf32 precision)
+  constexpr bool kCanSplit = sizeof(T) == 4 && S == 4 && NT != 4;
+  const bool split = kCanSplit && d.reduced && split_bf16_enabled() && (!g.wave || g.split);
+  auto kern = split ? bwd_fused_kernel<T, NT, S, BI, BJ, kCanSplit ? 4 : 2> : bwd_fused_kernel<T, NT, S, BI, BJ, 2>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   {
@@ -1237,6 +1265,12 @@ int launch_side_job(const SideJob &job, hipStream_t stream) {
   side_job_kernel<<<(unsigned)job.blocks, 256, 0, stream>>>(job);
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
+}
+
+// FGMS_SPLIT_BF16=0 keeps fp32 tensors on fp32 MFMAs in "tf32" mode too (for comparison).
+bool split_bf16_enabled() {
+  static const bool on = !(getenv("FGMS_SPLIT_BF16") && atoi(getenv("FGMS_SPLIT_BF16")) == 0);
+  return on;
 }
 
 bool mfma_gms_supported(const GmsArgs &a) { return shape_of(a).ok; }

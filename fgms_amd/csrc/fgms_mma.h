@@ -37,6 +37,18 @@ __device__ __forceinline__ float swap_with_neighbour(float v) {
       float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
 }
 
+// fp32 value as two bf16 numbers, x = hi + lo + O(2^-17 x) (see the split-bf16 kernels).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef int int2v __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void split_bf16(float x, __bf16 &hi, __bf16 &lo) {
+  hi = (__bf16)x;
+  const float h = (float)hi;
+  // (an infinite or NaN value stays in hi alone)
+  lo = (__bf16)(__builtin_fabsf(h) < __builtin_inff() ? x - h : 0.f);
+}
+
 // Re-lays the weights into per-lane MFMA fragment order in the stream's
 // workspace (see pack_weights_kernel) and returns the packed buffer.
 int pack_weights_any(const GmsArgs &a, int S, const void **packed);

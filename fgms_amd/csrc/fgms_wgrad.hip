@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
 }
 
 // The per-wave variant (wgrad_wave_body) in a launch of its own.
-template <typename T, int BI, int BJ>
+template <typename T, int BI, int BJ, bool SPLIT>
 __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     }
     block_x -= side.blocks;
   }
-  wgrad_wave_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, block_x, blockIdx.y);
+  wgrad_wave_body<T, BI, BJ, SPLIT>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, block_x, blockIdx.y);
 }
 
 // ---------------------------------------------------------------------------
@@ -296,11 +296,12 @@ int launch_wave(const WgradArgs &a, float *acc32) {
   WgradGeometry g;
   int rc = wgrad_geometry(a, &g);
   if (rc != FGMS_OK) return rc;
-  auto kern = wgrad_wave_kernel<T, BI, BJ>;
+  constexpr bool kCanSplit = sizeof(T) == 4;
+  auto kern = g.split ? wgrad_wave_kernel<T, BI, BJ, kCanSplit> : wgrad_wave_kernel<T, BI, BJ, false>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds));
   {
-    ProfileScope prof("wgrad_wave_kernel", a.stream);
+    ProfileScope prof(g.split ? "wgrad_wave_kernel(bf16x3)" : "wgrad_wave_kernel", a.stream);
     kern<<<dim3((unsigned)g.tiles + (unsigned)a.side.blocks, (unsigned)g.ty), kThreads, g.lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
         a.c_out, g.smap, a.side);
@@ -391,7 +392,10 @@ int wgrad_geometry(const WgradArgs &a, WgradGeometry *g, bool shares_grid) {
     const int sp = f16 ? WTW<__half>::stage_pairs : WTW<float>::stage_pairs;
     g->smap = choose_slices(a, g->ty, sp, (int64_t)num_cus() * 6);
     g->tiles = (int64_t)g->smap.slices * a.k_vol;
-    const size_t lds = 4 * (size_t)sp * ((bi * 32 + pad) + (bj * 32 + pad)) * esz;
+    // fp32 tensors whose caller allows tf32 precision: four 16-bit tiles per wave instead
+    g->split = !f16 && a.reduced && split_bf16_enabled();
+    const size_t lds = g->split ? 4 * (size_t)sp * 2 * ((bi * 32 + 16) + (bj * 32 + 16)) * 2
+                                : 4 * (size_t)sp * ((bi * 32 + pad) + (bj * 32 + pad)) * esz;
     const size_t red = 2 * (size_t)bi * bj * 16 * 64 * sizeof(float);
     g->lds = lds < red ? red : lds;
     return FGMS_OK;

@@ -93,7 +93,11 @@ template <> struct WTW<__half> { static constexpr int stage_pairs = 32; };
 template <> struct WTW<float> { static constexpr int stage_pairs = 16; };
 
 // (block_x, block_y): the workgroup's place in a grid of cells x tiles of dW[k]; 256 threads.
-template <typename T, int BI, int BJ>
+// SPLIT (fp32 tensors whose caller allows tf32 precision): the staged rows are split into
+// bf16 pairs, x = hi + lo, on their way to LDS -- four 16-bit tiles per wave, laid out like
+// the fp16 path's two -- and a product is three bf16 MFMAs, hi*hi + hi*lo + lo*hi, fed
+// through the same transposing LDS reads as fp16.
+template <typename T, int BI, int BJ, bool SPLIT = false>
 __device__ __forceinline__ void wgrad_wave_body(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
@@ -115,6 +119,11 @@ __device__ __forceinline__ void wgrad_wave_body(
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   T *x = reinterpret_cast<T *>(lds) + (size_t)wave * SP * (LDI + LDO);
   T *g = x + SP * LDI;
+  // SPLIT: 16-bit tiles with the fp16 path's row padding (32 bytes)
+  constexpr int LDIh = CI + 16, LDOh = CO + 16;
+  __half *xh = reinterpret_cast<__half *>(lds) + (size_t)wave * SP * 2 * (LDIh + LDOh);
+  __half *xl = xh + SP * LDIh, *gh = xl + SP * LDIh, *gl = gh + SP * LDOh;
+  static_assert(!SPLIT || (sizeof(T) == 4 && SP == 16), "split tiles: fp32 rows, one 16-pair MFMA step a stage");
 
   float16v acc[BI][BJ];
 #pragma unroll
@@ -153,18 +162,44 @@ __device__ __forceinline__ void wgrad_wave_body(
       gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
     }
   };
+  // SPLIT: chunk c (4 fp32 values) of a row -> 4 hi and 4 lo bf16; lane pairs hold neighbouring
+  // chunks and exchange halves, so the even lane writes 8 hi values and the odd one 8 lo
+  // values, 16 bytes each
+  auto store_split = [&](__half *hi_tile, __half *lo_tile, int ld, int row, int c, const int4v &raw, bool valid) {
+    const bool odd = lane & 1;
+    const float4v v = valid ? __builtin_bit_cast(float4v, raw) : float4v{0.f, 0.f, 0.f, 0.f};
+    bf16x4 hi, lo;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      __bf16 h, l;
+      split_bf16(v[q], h, l);
+      hi[q] = h;
+      lo[q] = l;
+    }
+    const int2v h2 = __builtin_bit_cast(int2v, hi), l2 = __builtin_bit_cast(int2v, lo);
+    const int got0 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[0] : l2[0])));
+    const int got1 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[1] : l2[1])));
+    if (odd) *reinterpret_cast<int4v *>(lo_tile + row * ld + (c - 1) * 4) = int4v{got0, got1, l2[0], l2[1]};
+    else *reinterpret_cast<int4v *>(hi_tile + row * ld + c * 4) = int4v{h2[0], h2[1], got0, got1};
+  };
   auto store_rows = [&](int st) {     // st: the stage the rows in flight belong to
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int e = lane + 64 * i;
-      *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
-          st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
+      if constexpr (SPLIT)
+        store_split(xh, xl, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count);
+      else
+        *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
+            st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int e = lane + 64 * i;
-      *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
-          st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
+      if constexpr (SPLIT)
+        store_split(gh, gl, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count);
+      else
+        *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
+            st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
     }
   };
   auto wave_fence = [] {
@@ -183,6 +218,27 @@ __device__ __forceinline__ void wgrad_wave_body(
     __builtin_amdgcn_sched_barrier(0);   // (rows first, then indices, both before the MFMAs:
     load_idx(st + 8);                    //  the wait for the rows then leaves the indices in flight)
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (SPLIT) {
+      bf16x8 ah[BI], al[BI], bh[BJ], bl[BJ];
+#pragma unroll
+      for (int ti = 0; ti < BI; ++ti) {
+        ah[ti] = __builtin_bit_cast(bf16x8, tr_frag(xh, LDIh, 0, ti * 32, lane));
+        al[ti] = __builtin_bit_cast(bf16x8, tr_frag(xl, LDIh, 0, ti * 32, lane));
+      }
+#pragma unroll
+      for (int tj = 0; tj < BJ; ++tj) {
+        bh[tj] = __builtin_bit_cast(bf16x8, tr_frag(gh, LDOh, 0, tj * 32, lane));
+        bl[tj] = __builtin_bit_cast(bf16x8, tr_frag(gl, LDOh, 0, tj * 32, lane));
+      }
+#pragma unroll
+      for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < BJ; ++tj) {
+          acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ti], bh[tj], acc[ti][tj], 0, 0, 0);
+          acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ti], bl[tj], acc[ti][tj], 0, 0, 0);
+          acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ti], bh[tj], acc[ti][tj], 0, 0, 0);
+        }
+    } else {
 #pragma unroll
     for (int ks = 0; ks < SP / KP; ++ks) {
       const int p0 = ks * KP;
@@ -213,6 +269,7 @@ __device__ __forceinline__ void wgrad_wave_body(
               acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ti], b[tj], acc[ti][tj], 0, 0, 0);
         }
       }
+    }
     }
     wave_fence();                   // the tile is rewritten at the top of the loop
     st += 4;
@@ -461,6 +518,7 @@ struct WgradGeometry {
   int ty;          // grid y: BI*32 x BJ*32 tiles of dW[k]
   int bi, bj;
   bool wave;       // wgrad_wave_body, else wgrad_wg_body
+  bool split;      // wgrad_wave_body in split bf16
   size_t lds;      // dynamic LDS
 };
 // shares_grid: the launch also holds the input gradient's workgroups.

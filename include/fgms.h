@@ -23,10 +23,11 @@
  *   - arch80: for FGMS_F32, non-zero = "tf32 mode" in the reference
  *     (backend/spconv.cu:67-68,213): the products may be rounded to tf32
  *     precision, the sums are fp32.  gfx950 has no tf32 matrix instruction;
- *     the forward pass with a plan then multiplies in split bf16 (every value
+ *     with a plan the forward pass, the input gradient and (for tiles of dW up
+ *     to 64 x 64) the weight gradient then multiply in split bf16 (every value
  *     as hi + lo, three 16-bit MFMAs per product: about 2^-16 relative error,
- *     finer than tf32, at twice the speed of the fp32 kernels).  Everything
- *     else, and arch80 = 0, runs the fp32 MFMA kernels.
+ *     finer than tf32, at about twice the speed of the fp32 kernels).
+ *     Everything else, and arch80 = 0, runs the fp32 MFMA kernels.
  *   - stream: a hipStream_t (NULL = the null stream).  All work is enqueued on
  *     it; calls return without waiting for the GPU, as the reference's do.
  *   - plan: optional (NULL allowed) handle from fgms_plan_create for the same
@@ -107,8 +108,10 @@ int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz,
 /*
  * Replaces ConvolutionBackward  (backend/spconv.cu:414-571; pybind name
  * fgms_bwd_cuda, backend/pybind_cuda.cpp:10): input gradient and weight
- * gradient, both accumulated into caller-zeroed buffers.  separate_mid and
- * arch80 are accepted and ignored, as in the reference.  (The reference launches
+ * gradient, both accumulated into caller-zeroed buffers.  separate_mid is
+ * accepted and ignored, as in the reference; arch80 is ignored there because its
+ * backward pass of fp32 tensors is always tf32 (backend/spconv.cu:551-569), here
+ * it allows that precision as in the forward pass (see above).  (The reference launches
  * the input gradient, then the weight gradient; the two do not depend on each
  * other, and with a plan this library runs the workgroups of both in one launch,
  * followed for fp16 by a small one that rounds the weight gradient's fp32 sums.)

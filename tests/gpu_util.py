@@ -53,7 +53,7 @@ def run_fwd(capi, D, fused=True, separate_mid=False, arch80=False, plan=None, ou
     return out.cpu().numpy()
 
 
-def run_bwd(capi, D, plan=None, split=False):
+def run_bwd(capi, D, plan=None, split=False, arch80=False):
     gi = torch.zeros(D["n_in"], D["c_in"], dtype=D["in_feats"].dtype, device="cuda")
     gw = torch.zeros_like(D["kernel"])
     if split:
@@ -61,6 +61,6 @@ def run_bwd(capi, D, plan=None, split=False):
         capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
     else:
         capi.bwd(D["out_grad"], D["in_feats"], D["kernel"], 0, gi, gw, D["kpos"], None,
-                 D["imap"], D["omap"], False, False, plan=plan)
+                 D["imap"], D["omap"], False, arch80, plan=plan)
     torch.cuda.synchronize()
     return gi.cpu().numpy(), gw.cpu().numpy()
