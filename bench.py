@@ -33,6 +33,8 @@ WORKLOADS = {
     "cfg2-indoor200k-k27-64x64-fp16-fwd": (2, "fp16", ("fwd",)),
     "cfg2-indoor200k-k27-64x64-fp32-fwd": (2, None, ("fwd",)),
     "cfg2-indoor200k-k27-64x64-tf32-fwd": (2, "tf32", ("fwd",)),
+    "cfg2-indoor200k-k27-64x64-tf32-fwd+dgrad+wgrad": (2, "tf32", ("fwd", "dgrad", "wgrad")),
+    "cfg2-indoor200k-k27-64x64-fp32-fwd+dgrad+wgrad": (2, None, ("fwd", "dgrad", "wgrad")),
     "cfg1-planes20k-k27-32x32-fp32-fwd+dgrad+wgrad": (1, None, ("fwd", "dgrad", "wgrad")),
     "cfg3-lidar120k-k27-128x128-fp16-fwd+dgrad+wgrad": (3, None, ("fwd", "dgrad", "wgrad")),
     "cfg4-down-k8-64x128-fp16-fwd+dgrad+wgrad": (4, None, ("fwd", "dgrad", "wgrad")),

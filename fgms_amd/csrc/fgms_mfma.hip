@@ -1095,8 +1095,8 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
       wgrad_wave_body<T, BI, BJ, RAWD == 4>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap,
                                             j % wgrad_x, j / wgrad_x);
     else
-      wgrad_wg_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, j % wgrad_x,
-                               j / wgrad_x);
+      wgrad_wg_body<T, BI, BJ, RAWD == 4>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap,
+                                          j % wgrad_x, j / wgrad_x);
   }
 }
 
@@ -1126,12 +1126,12 @@ int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArg
   // RAWD: how the input gradient reads the weights (2: as they lie; 4: also split into bf16
   // pairs, for fp32 tensors whose caller allows tf32 precision)
   constexpr bool kCanSplit = sizeof(T) == 4 && S == 4 && NT != 4;
-  const bool split = kCanSplit && d.reduced && split_bf16_enabled() && (!g.wave || g.split);
+  const bool split = kCanSplit && d.reduced && split_bf16_enabled() && g.split;
   auto kern = split ? bwd_fused_kernel<T, NT, S, BI, BJ, kCanSplit ? 4 : 2> : bwd_fused_kernel<T, NT, S, BI, BJ, 2>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   {
-    ProfileScope prof("bwd_fused_kernel", d.stream);
+    ProfileScope prof(split ? "bwd_fused_kernel(bf16x3)" : "bwd_fused_kernel", d.stream);
     kern<<<row_x * row_y * row_z + (unsigned)(g.tiles * g.ty), kThreads, lds, d.stream>>>(
         (const T *)d.src, (const T *)d.w, (T *)d.dst, p->nbr_in, p->mask_in, p->perm_in, p->tile_in,
         (int)d.n_dst, d.k_vol, d.c_in, d.c_out, part_stages, (const T *)w.in, acc32, w.kpos, w.imap, w.omap,

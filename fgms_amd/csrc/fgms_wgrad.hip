@@ -32,7 +32,7 @@ constexpr int kThreads = 256;
 constexpr int kSkinnyThreads = 256;    // the skinny weight-gradient kernel
 
 // The workgroup-level variant (wgrad_wg_body) in a launch of its own.
-template <typename T, int BI, int BJ>
+template <typename T, int BI, int BJ, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void wgrad_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(
     }
     block_x -= side.blocks;
   }
-  wgrad_wg_body<T, BI, BJ>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, block_x, blockIdx.y);
+  wgrad_wg_body<T, BI, BJ, SPLIT>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, block_x, blockIdx.y);
 }
 
 // The per-wave variant (wgrad_wave_body) in a launch of its own.
@@ -278,11 +278,12 @@ int launch(const WgradArgs &a, float *acc32) {
   WgradGeometry g;
   int rc = wgrad_geometry(a, &g);
   if (rc != FGMS_OK) return rc;
-  auto kern = wgrad_kernel<T, BI, BJ>;
+  constexpr bool kCanSplit = sizeof(T) == 4;
+  auto kern = g.split ? wgrad_kernel<T, BI, BJ, kCanSplit> : wgrad_kernel<T, BI, BJ, false>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds));
   {
-    ProfileScope prof("wgrad_kernel", a.stream);
+    ProfileScope prof(g.split ? "wgrad_kernel(bf16x3)" : "wgrad_kernel", a.stream);
     kern<<<dim3((unsigned)g.tiles + (unsigned)a.side.blocks, (unsigned)g.ty), kThreads, g.lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
         a.c_out, g.smap, a.side);
@@ -416,7 +417,9 @@ int wgrad_geometry(const WgradArgs &a, WgradGeometry *g, bool shares_grid) {
     g->smap = choose_slices(a, g->ty, sp, (int64_t)num_cus() * 4);
     g->tiles = (int64_t)g->smap.slices * a.k_vol;
   }
-  g->lds = 2 * (size_t)sp * ((bi * 32 + pad) + (bj * 32 + pad)) * esz;
+  g->split = !f16 && a.reduced && split_bf16_enabled();
+  g->lds = g->split ? 2 * (size_t)sp * 2 * ((bi * 32 + 16) + (bj * 32 + 16)) * 2
+                    : 2 * (size_t)sp * ((bi * 32 + pad) + (bj * 32 + pad)) * esz;
   return FGMS_OK;
 }
 

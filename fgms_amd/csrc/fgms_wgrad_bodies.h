@@ -82,6 +82,29 @@ __device__ __forceinline__ bool locate_slice(const int32_t *__restrict__ kpos, c
   return count > 0;
 }
 
+// Split staging (fp32 rows whose caller allows tf32 precision): chunk c (4 fp32 values) of a
+// staged row becomes 4 hi and 4 lo bf16 values in two 16-bit tiles laid out like the fp16
+// path's.  Lane pairs hold neighbouring chunks and exchange halves, so the even lane writes
+// 8 hi values and the odd one 8 lo values, 16 bytes each.
+__device__ __forceinline__ void store_split_chunk(__half *hi_tile, __half *lo_tile, int ld, int row, int c,
+                                                  const int4v &raw, bool valid, int lane) {
+  const bool odd = lane & 1;
+  const float4v v = valid ? __builtin_bit_cast(float4v, raw) : float4v{0.f, 0.f, 0.f, 0.f};
+  bf16x4 hi, lo;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    __bf16 h, l;
+    split_bf16(v[q], h, l);
+    hi[q] = h;
+    lo[q] = l;
+  }
+  const int2v h2 = __builtin_bit_cast(int2v, hi), l2 = __builtin_bit_cast(int2v, lo);
+  const int got0 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[0] : l2[0])));
+  const int got1 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[1] : l2[1])));
+  if (odd) *reinterpret_cast<int4v *>(lo_tile + row * ld + (c - 1) * 4) = int4v{got0, got1, l2[0], l2[1]};
+  else *reinterpret_cast<int4v *>(hi_tile + row * ld + c * 4) = int4v{h2[0], h2[1], got0, got1};
+}
+
 // Variant for dW tiles up to 64 x 64: every wave stages its own pairs in its own
 // LDS region and multiplies them into a private copy of the whole tile, so the
 // pair loop has no workgroup barrier at all (the four waves take the chunk's
@@ -162,32 +185,12 @@ __device__ __forceinline__ void wgrad_wave_body(
       gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
     }
   };
-  // SPLIT: chunk c (4 fp32 values) of a row -> 4 hi and 4 lo bf16; lane pairs hold neighbouring
-  // chunks and exchange halves, so the even lane writes 8 hi values and the odd one 8 lo
-  // values, 16 bytes each
-  auto store_split = [&](__half *hi_tile, __half *lo_tile, int ld, int row, int c, const int4v &raw, bool valid) {
-    const bool odd = lane & 1;
-    const float4v v = valid ? __builtin_bit_cast(float4v, raw) : float4v{0.f, 0.f, 0.f, 0.f};
-    bf16x4 hi, lo;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      __bf16 h, l;
-      split_bf16(v[q], h, l);
-      hi[q] = h;
-      lo[q] = l;
-    }
-    const int2v h2 = __builtin_bit_cast(int2v, hi), l2 = __builtin_bit_cast(int2v, lo);
-    const int got0 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[0] : l2[0])));
-    const int got1 = __builtin_bit_cast(int, swap_with_neighbour(__builtin_bit_cast(float, odd ? h2[1] : l2[1])));
-    if (odd) *reinterpret_cast<int4v *>(lo_tile + row * ld + (c - 1) * 4) = int4v{got0, got1, l2[0], l2[1]};
-    else *reinterpret_cast<int4v *>(hi_tile + row * ld + c * 4) = int4v{h2[0], h2[1], got0, got1};
-  };
   auto store_rows = [&](int st) {     // st: the stage the rows in flight belong to
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int e = lane + 64 * i;
       if constexpr (SPLIT)
-        store_split(xh, xl, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count);
+        store_split_chunk(xh, xl, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count, lane);
       else
         *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
             st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
@@ -196,7 +199,7 @@ __device__ __forceinline__ void wgrad_wave_body(
     for (int i = 0; i < NG; ++i) {
       const int e = lane + 64 * i;
       if constexpr (SPLIT)
-        store_split(gh, gl, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count);
+        store_split_chunk(gh, gl, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count, lane);
       else
         *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
             st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
@@ -330,7 +333,8 @@ template <int BI, int BJ> struct WaveGrid {
 // The workgroup-level weight-gradient kernel body (dW tiles wider than 64 x 64): the four
 // waves share the staged pairs and split the tile.  (block_x, block_y): the workgroup's
 // place in a grid of cells x tiles of dW[k]; 256 threads.
-template <typename T, int BI, int BJ>
+// SPLIT: as in wgrad_wave_body (fp32 rows staged as hi / lo bf16 tiles, three bf16 MFMAs a product).
+template <typename T, int BI, int BJ, bool SPLIT = false>
 __device__ __forceinline__ void wgrad_wg_body(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
@@ -351,6 +355,11 @@ __device__ __forceinline__ void wgrad_wg_body(
   // global loads in flight.)
   T *const stage0 = reinterpret_cast<T *>(lds);
   constexpr int kBufElems = SP * (LDI + LDO);
+  // SPLIT: a buffer holds four 16-bit tiles, x hi, x lo, g hi, g lo, rows padded as in the fp16 path
+  constexpr int LDIh = CI + 16, LDOh = CO + 16;
+  constexpr int kBufHalfs = SP * 2 * (LDIh + LDOh);
+  __half *const stage0h = reinterpret_cast<__half *>(lds);
+  static_assert(!SPLIT || (sizeof(T) == 4 && G::WK == 1 && SP % 16 == 0), "split tiles: fp32 rows, whole 16-pair steps");
 
   int k, first, count;
   if (!locate_slice(kpos, smap, k_vol, block_x, k, first, count)) return;
@@ -404,17 +413,54 @@ __device__ __forceinline__ void wgrad_wg_body(
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int e = tid + kThreads * i;
-      *reinterpret_cast<int4v *>(stage0 + buf * kBufElems + (e / NCI) * LDI + (e % NCI) * E) =
-          st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
+      if constexpr (SPLIT) {
+        __half *xh = stage0h + buf * kBufHalfs;
+        store_split_chunk(xh, xh + SP * LDIh, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count, lane);
+      } else {
+        *reinterpret_cast<int4v *>(stage0 + buf * kBufElems + (e / NCI) * LDI + (e % NCI) * E) =
+            st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
+      }
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int e = tid + kThreads * i;
-      *reinterpret_cast<int4v *>(stage0 + buf * kBufElems + SP * LDI + (e / NCO) * LDO + (e % NCO) * E) =
-          st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
+      if constexpr (SPLIT) {
+        __half *gh = stage0h + buf * kBufHalfs + SP * 2 * LDIh;
+        store_split_chunk(gh, gh + SP * LDOh, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count, lane);
+      } else {
+        *reinterpret_cast<int4v *>(stage0 + buf * kBufElems + SP * LDI + (e / NCO) * LDO + (e % NCO) * E) =
+            st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
+      }
     }
   };
   auto multiply = [&](int cur) {
+    if constexpr (SPLIT) {
+      const __half *xh = stage0h + cur * kBufHalfs, *xl = xh + SP * LDIh;
+      const __half *gh = xl + SP * LDIh, *gl = gh + SP * LDOh;
+#pragma unroll
+      for (int p0 = 0; p0 < SP; p0 += 16) {
+        bf16x8 ah[G::TI], al[G::TI], bh[G::TJ], bl[G::TJ];
+#pragma unroll
+        for (int ti = 0; ti < G::TI; ++ti) {
+          ah[ti] = __builtin_bit_cast(bf16x8, tr_frag(xh, LDIh, p0, (wi * G::TI + ti) * 32, lane));
+          al[ti] = __builtin_bit_cast(bf16x8, tr_frag(xl, LDIh, p0, (wi * G::TI + ti) * 32, lane));
+        }
+#pragma unroll
+        for (int tj = 0; tj < G::TJ; ++tj) {
+          bh[tj] = __builtin_bit_cast(bf16x8, tr_frag(gh, LDOh, p0, (wj * G::TJ + tj) * 32, lane));
+          bl[tj] = __builtin_bit_cast(bf16x8, tr_frag(gl, LDOh, p0, (wj * G::TJ + tj) * 32, lane));
+        }
+#pragma unroll
+        for (int ti = 0; ti < G::TI; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < G::TJ; ++tj) {
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ti], bh[tj], acc[ti][tj], 0, 0, 0);
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ti], bl[tj], acc[ti][tj], 0, 0, 0);
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ti], bh[tj], acc[ti][tj], 0, 0, 0);
+          }
+      }
+      return;
+    }
     const T *x = stage0 + cur * kBufElems, *g = x + SP * LDI;
 #pragma unroll
     for (int ks = wk; ks < SP / KP; ks += G::WK) {

@@ -409,12 +409,12 @@ def test_tf32_mode_multiplies_in_split_bf16(capi, oracle, shape):
 
 
 @pytest.mark.parametrize("kind", ["subm", "down"])
-@pytest.mark.parametrize("shape", [(64, 64), (32, 64), (96, 32), (64, 128)], ids=lambda s: "%dx%d" % s)
+@pytest.mark.parametrize("shape", [(64, 64), (32, 64), (96, 32), (64, 128), (128, 128)], ids=lambda s: "%dx%d" % s)
 def test_tf32_mode_backward_in_split_bf16(capi, oracle, shape, kind):
     """fgms_bwd of fp32 tensors with arch80 set (the reference's backward is tf32 whenever the
-    tensors are fp32, backend/spconv.cu:551-569): the input gradient and, for dW tiles up to
-    64 x 64, the weight gradient multiply in split bf16.  Both stay within 1e-4 of the
-    result's rms (tf32 would be allowed 1e-2), on two calls in a row."""
+    tensors are fp32, backend/spconv.cu:551-569): the input gradient and the weight gradient
+    (per-wave and workgroup-level kernel bodies alike) multiply in split bf16.  Both stay
+    within 1e-4 of the result's rms (tf32 would be allowed 1e-2), on two calls in a row."""
     L = layer(29, shape[0], shape[1], np.float32, kind)
     D = G.to_dev(L)
     capi.set_kernel_policy(4)
@@ -429,8 +429,8 @@ def test_tf32_mode_backward_in_split_bf16(capi, oracle, shape, kind):
             G.assert_close(got, want, "tf32", "tf32-mode " + what)
             rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
             assert np.abs(got - want).max() <= 1e-4 * rms, what
-    # the split path is the one that ran: the input gradient differs from the fp32 kernels' in its last bits
-    assert not np.array_equal(gi, exact_gi)
+    # the split path is the one that ran: both gradients differ from the fp32 kernels' in their last bits
+    assert not np.array_equal(gi, exact_gi) and not np.array_equal(gw, exact_gw)
     G.assert_close(exact_gi, want_gi, "fp32", "fp32 dgrad")
     G.assert_close(exact_gw, want_gw, "fp32", "fp32 wgrad")
     plan.close()
