@@ -82,6 +82,18 @@ __device__ __forceinline__ void load_weights(int4v *__restrict__ w_lds,
   }
 }
 
+// The same for split weights (pack_weights_bf3_kernel): per (slab, k-step) NT * 128 chunks.
+template <int NT>
+__device__ __forceinline__ void load_weights_bf3(int4v *__restrict__ w_lds,
+                                                 const int4v *__restrict__ packed_k, int slabs, int nts,
+                                                 int nt0) {
+  const int n = slabs * 2 * NT * 128;
+  for (int i = threadIdx.x; i < n; i += kThreads) {
+    const int q = i / (NT * 128), rem = i % (NT * 128);
+    w_lds[i] = packed_k[((size_t)q * nts + nt0) * 128 + rem];
+  }
+}
+
 // acc[mt][nt] += A(slab) x W(slab).
 template <typename T, int NT, int S>
 __device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
@@ -281,11 +293,12 @@ __device__ __forceinline__ void mma_slab_bf3t(float16v (&acc)[2][NT], const int4
 
 // Split weights in the order mma_slab_bf3 reads them: chunk
 //   ((((k * slabs + slab) * 2 + s) * nts + nt) * 2 + part) * 64 + lane
-// holds the 8 values W[k][slab*32 + s*16 + (lane/32)*8 + 0..7][nt*32 + lane%32], hi (part 0)
+// holds the 8 values op(W[k])[slab*32 + s*16 + (lane/32)*8 + 0..7][nt*32 + lane%32], hi (part 0)
 // or lo (part 1).  One thread per chunk pair.
 __global__ void pack_weights_bf3_kernel(const float *__restrict__ w, int4v *__restrict__ packed,
-                                        int k_vol, int c_in, int c_out) {
-  const int slabs = c_in / 32, nts = c_out / 32;
+                                        int k_vol, int c_in, int c_out, bool transpose) {
+  // (transpose: the input gradient's view, W[k]^T -- source channels are the columns of W[k])
+  const int slabs = (transpose ? c_out : c_in) / 32, nts = (transpose ? c_in : c_out) / 32;
   const size_t total = (size_t)k_vol * slabs * 2 * nts * 64;
   for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
        t += (size_t)gridDim.x * blockDim.x) {
@@ -300,7 +313,7 @@ __global__ void pack_weights_bf3_kernel(const float *__restrict__ w, int4v *__re
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       __bf16 h, l;
-      split_bf16(w[((size_t)k * c_in + cs0 + e) * c_out + cd], h, l);
+      split_bf16(transpose ? w[((size_t)k * c_in + cd) * c_out + cs0 + e] : w[((size_t)k * c_in + cs0 + e) * c_out + cd], h, l);
       hi[e] = h;
       lo[e] = l;
     }
@@ -559,7 +572,9 @@ __device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (
 
 // ---------------------------------------------------------------------------
 // Pair-stationary kernel.
-template <typename T, int NT, int S>
+// SPLIT: fp32 tensors whose caller allows tf32 precision, products in split bf16 (see
+// mma_slab_bf3); `packed` from pack_weights_bf3_kernel.
+template <typename T, int NT, int S, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ gmap,
@@ -593,7 +608,10 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
     }
     if (k != cur_k) {  // uniform over the workgroup
       __syncthreads();
-      load_weights<NT>(w_lds, reinterpret_cast<const int4v *>(packed) + packed_per_k * k, qs, nts, nt0);
+      if constexpr (SPLIT)
+        load_weights_bf3<NT>(w_lds, reinterpret_cast<const int4v *>(packed) + packed_per_k * k, slabs, nts, nt0);
+      else
+        load_weights<NT>(w_lds, reinterpret_cast<const int4v *>(packed) + packed_per_k * k, qs, nts, nt0);
       __syncthreads();
       cur_k = k;
     }
@@ -618,10 +636,12 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
     int gsel[2 * S];
     gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
     for (int slab = 0; slab < slabs; ++slab) {
-      gather_commit<S>(a_lds, v, gsel, lane);
+      if constexpr (SPLIT) gather_commit_bf3(a_lds, v, gsel, lane);
+      else gather_commit<S>(a_lds, v, gsel, lane);
       wave_lds_fence();
       if (slab + 1 < slabs) gather_issue<T, S>(v, gsel, gidx, src, c_src, slab + 1, lane);   // under the MFMAs
-      mma_slab<T, NT, S>(acc, a_lds, w_lds, slab, lane);
+      if constexpr (SPLIT) mma_slab_bf3<NT>(acc, a_lds, w_lds + slab * (2 * NT * 128), lane);
+      else mma_slab<T, NT, S>(acc, a_lds, w_lds, slab, lane);
       wave_lds_fence();
     }
     write_tile<T, NT, true>(acc, dst, sidx, c_dst, nt0 * 32, lane);
@@ -959,8 +979,23 @@ int pack_weights(const GmsArgs &a, const Shape &s, const T **packed) {
 template <typename T, int NT, int S>
 int launch_pairs(const GmsArgs &a, const Shape &s) {
   const T *packed = nullptr;
-  int rc = pack_weights<T>(a, s, &packed);
-  if (rc != FGMS_OK) return rc;
+  // fp32 tensors whose caller allows tf32 precision: products in split bf16
+  constexpr bool kCanSplit = sizeof(T) == 4 && S == 4;
+  const bool split = kCanSplit && a.reduced && split_bf16_enabled();
+  if (split) {
+    void *ws = nullptr;
+    const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+    int rc = workspace_get(a.stream, 0, n * sizeof(float), &ws);
+    if (rc != FGMS_OK) return rc;
+    size_t blocks = (n / 8 + 255) / 256;
+    pack_weights_bf3_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, a.stream>>>(
+        (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out, a.transpose_w);
+    FGMS_HIP_TRY(hipGetLastError());
+    packed = (const T *)ws;
+  } else {
+    int rc = pack_weights<T>(a, s, &packed);
+    if (rc != FGMS_OK) return rc;
+  }
   const bool dense = a.dense_k >= 0;
   const int64_t tiles = dense ? (a.n_dense + kTileRows - 1) / kTileRows
                               : (a.n_pairs + kTileRows - 1) / kTileRows + a.k_vol;
@@ -968,11 +1003,13 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   const int64_t want_wgs = (int64_t)num_cus() * 8;
   const int tiles_per_wg = (int)((tiles + want_wgs - 1) / want_wgs);
   const unsigned gx = (unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg);
-  auto kern = gms_pairs_kernel<T, NT, S>;
+  auto kern = split ? gms_pairs_kernel<T, NT, S, kCanSplit> : gms_pairs_kernel<T, NT, S, false>;
   FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)s.lds_bytes));
   {
-    ProfileScope prof(a.transpose_w ? "gms_pairs_kernel(dgrad)" : "gms_pairs_kernel(fwd)", a.stream);
+    ProfileScope prof(split ? (a.transpose_w ? "gms_pairs_kernel(dgrad, bf16x3)" : "gms_pairs_kernel(fwd, bf16x3)")
+                            : (a.transpose_w ? "gms_pairs_kernel(dgrad)" : "gms_pairs_kernel(fwd)"),
+                      a.stream);
     kern<<<dim3(gx, (unsigned)(s.c_dst / (32 * NT))), kThreads, s.lds_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, a.kpos, a.gmap, a.smap, a.k_vol, s.c_src, s.c_dst,
         tiles_per_wg, a.dense_k, (int)a.n_dense);
@@ -1015,7 +1052,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
     if (rc != FGMS_OK) return rc;
     size_t blocks = (n / 8 + 255) / 256;
     pack_weights_bf3_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, a.stream>>>(
-        (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out);
+        (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out, false);
     FGMS_HIP_TRY(hipGetLastError());
     packed = (const T *)ws;
     raw = 3;

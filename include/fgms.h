@@ -23,8 +23,9 @@
  *   - arch80: for FGMS_F32, non-zero = "tf32 mode" in the reference
  *     (backend/spconv.cu:67-68,213): the products may be rounded to tf32
  *     precision, the sums are fp32.  gfx950 has no tf32 matrix instruction;
- *     with a plan the forward pass, the input gradient and the weight
- *     gradient then multiply in split bf16 (every value
+ *     the forward pass, the input gradient and the weight gradient (the MFMA
+ *     kernels: channel counts that are multiples of 32) then multiply in split
+ *     bf16 (every value
  *     as hi + lo, three 16-bit MFMAs per product: about 2^-16 relative error,
  *     finer than tf32, at about twice the speed of the fp32 kernels).
  *     Everything else, and arch80 = 0, runs the fp32 MFMA kernels.

@@ -435,3 +435,37 @@ def test_tf32_mode_backward_in_split_bf16(capi, oracle, shape, kind):
     G.assert_close(exact_gw, want_gw, "fp32", "fp32 wgrad")
     plan.close()
     capi.set_kernel_policy(0)
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (96, 32), (256, 256)], ids=lambda s: "%dx%d" % s)
+def test_tf32_mode_without_a_plan(capi, oracle, shape):
+    """The pair-stationary kernels (calls without a plan) multiply in split bf16 as well,
+    forward (also with the centre offset taken apart) and backward."""
+    L = layer(37, shape[0], shape[1], np.float32)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(0)
+    args = (L["knnz"], L["imap"], L["omap"])
+    want = oracle.np_fwd(L["in_feats"], L["kernel"], *args, L["n_out"])
+    capi.profile_reset()
+    capi.profile_enable(True)
+    out = G.run_fwd(capi, D, fused=True, arch80=True, plan=None)
+    gi, gw = G.run_bwd(capi, D, plan=None, arch80=True)
+    capi.profile_enable(False)
+    names = {n for n, _ in capi.profile_records()}
+    capi.profile_reset()
+    assert {"gms_pairs_kernel(fwd, bf16x3)", "gms_pairs_kernel(dgrad, bf16x3)"} <= names, names
+    for got, ref, what in ((out, want, "fwd"),
+                           (gi, oracle.np_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"]), "dgrad"),
+                           (gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"]), "wgrad")):
+        G.assert_close(got, ref, "tf32", "tf32-mode " + what)
+        assert np.abs(got - ref).max() <= 1e-4 * float(np.sqrt(np.mean(ref.astype(np.float64) ** 2))), what
+    # the centre offset left out of the map and added as a dense product (separate_mid)
+    rng = np.random.default_rng(38)
+    vox = cloud(38)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vox, vox, clouds.offsets_cube(3), skip_offset=13)
+    Ls = clouds.make_layer(rng, imap, omap, knnz, kpos, len(vox), len(vox), shape[0], shape[1], np.float32)
+    Ds = G.to_dev(Ls)
+    ref = oracle.np_fwd(Ls["in_feats"], Ls["kernel"], knnz, imap, omap, len(vox), precompute=True)
+    for fused in (True, False):
+        G.assert_close(G.run_fwd(capi, Ds, fused=fused, separate_mid=True, arch80=True, plan=None), ref, "tf32",
+                       "tf32-mode forward, centre apart")
