@@ -130,6 +130,15 @@ struct Plan {
   // (64-row block, offset) combinations with at least one pair: the output-stationary
   // kernels run stages * 64 row slots for n_pairs pairs
   int stages_out, stages_in;
+  // Pair view, kept for maps that leave most row slots of the output-stationary kernels
+  // empty (scattered clouds): the pair lists with every offset's run padded to a multiple
+  // of 64 (padding = -1), so that a 64-row block of pv_in / pv_out belongs to one offset,
+  // bit k of pv_mask[b] says which.  The output-stationary kernel walks these "virtual
+  // rows" like a plan whose rows have one neighbour each and adds its results with
+  // atomics.  nullptr: not built.
+  int32_t *pv_in, *pv_out;        // [pv_rows]
+  unsigned long long *pv_mask;    // [pv_rows / 64]
+  int64_t pv_rows;                // a multiple of 256
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -177,6 +186,9 @@ bool small_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_small_gms(const GmsArgs &a, const Plan *p);
 bool planned_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_planned_gms(const GmsArgs &a, const Plan *p);
+// The same kernel over the plan's pair view (no wasted row slots, atomic adds).
+bool pair_view_gms_supported(const GmsArgs &a, const Plan *p);
+int launch_pair_view_gms(const GmsArgs &a, const Plan *p);
 int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
                      const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
                      int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,

@@ -478,6 +478,28 @@ __device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__
           for (int j = 0; j < 4; ++j)
             stage[(g * 8 + h * 4 + j) * COLS + nt * 32 + col] = acc[mt][nt][(g0 + g) * 4 + j];
       wave_lds_fence();
+      if constexpr (ATOMIC) {
+        // Other workgroups add to the same rows.  An atomic instruction costs by the cache
+        // lines it touches, so neighbouring lanes take neighbouring 4-byte words of a row:
+        // one instruction covers 256 contiguous bytes.
+        constexpr int WORDS = sizeof(T) == 4 ? COLS : COLS / 2;      // 4-byte words per row
+#pragma unroll
+        for (int q = 0; q < R * WORDS / 64; ++q) {
+          const int e = q * 64 + lane;
+          const int r = e / WORDS, c = e % WORDS;
+          const int row = rows[p * R + r];
+          if constexpr (sizeof(T) == 4) {
+            const float v = stage[r * COLS + c];
+            if (row >= 0) atomic_add(reinterpret_cast<float *>(dst) + (size_t)row * c_dst + cd0 + c, v);
+          } else {
+            const float2 v = *reinterpret_cast<const float2 *>(stage + r * COLS + 2 * c);
+            if (row >= 0)
+              atomic_add_pk(reinterpret_cast<__half *>(dst) + (size_t)row * c_dst + cd0 + 2 * c, v.x, v.y);
+          }
+        }
+        wave_lds_fence();
+        continue;
+      }
       float4v part[IT];
       int row[IT];
 #pragma unroll
@@ -486,21 +508,7 @@ __device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__
         part[it] = *reinterpret_cast<const float4v *>(stage + (e / CH) * COLS + (e % CH) * 4);
         row[it] = rows[p * R + e / CH];
       }
-      if constexpr (ATOMIC) {
-        // another workgroup adds its share of the offsets to the same rows
-#pragma unroll
-        for (int it = 0; it < IT; ++it) {
-          if (row[it] < 0) continue;
-          T *p = dst + (size_t)row[it] * c_dst + cd0 + ((it * 64 + lane) % CH) * 4;
-          if constexpr (sizeof(T) == 4) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) atomic_add(reinterpret_cast<float *>(p) + q, part[it][q]);
-          } else {
-            atomic_add_pk(reinterpret_cast<__half *>(p), part[it][0], part[it][1]);
-            atomic_add_pk(reinterpret_cast<__half *>(p) + 2, part[it][2], part[it][3]);
-          }
-        }
-      } else if constexpr (sizeof(T) == 4) {
+      if constexpr (sizeof(T) == 4) {
         float4v old[IT];
 #pragma unroll
         for (int it = 0; it < IT; ++it)
@@ -671,9 +679,13 @@ __device__ __forceinline__ void gms_rows_body(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
-    int c_src, int c_dst, int part_stages, int block_x, int block_y, int block_z, int grid_z) {
+    int c_src, int c_dst, int part_stages, int block_x, int block_y, int block_z, int grid_z,
+    int pair_view = 0) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
+  // pair view: `nbr` is one list of source rows for all offsets (a 64-row block belongs to
+  // the one offset its mask names), `perm` the destination rows; results are added atomically
+  const size_t nbr_stride = pair_view ? 0 : (size_t)n_dst;
   constexpr int WCH = S * NT * 64;                        // 16-byte chunks of one stage's weights
   constexpr int NW = (WCH + kThreads - 1) / kThreads;     // ... per thread
   extern __shared__ int4v lds[];
@@ -708,7 +720,7 @@ __device__ __forceinline__ void gms_rows_body(
   // start of a launch every workgroup walks this chain of dependent loads at the same time
   // and nothing else covers it (0.4 us of a 46 us launch)
   int g_first = -1;
-  if (k_first >= 0 && in_range) g_first = nbr[(size_t)k_first * n_dst + my_row];
+  if (k_first >= 0 && in_range) g_first = nbr[(size_t)k_first * nbr_stride + my_row];
   didx[lane] = in_range ? (perm ? perm[my_row] : my_row) : -1;   // my_row is a position in the plan's row order
 
   // which offsets touch this wave's rows / this workgroup's rows (from the plan)
@@ -729,7 +741,7 @@ __device__ __forceinline__ void gms_rows_body(
   }
   // grid_z > 1: a tile is shared by up to grid_z workgroups, each takes a run
   // of the tile's offsets and adds its partial result with atomics.
-  bool shared_tile = false;
+  bool shared_tile = pair_view != 0;
   if (grid_z > 1) {
     const int n_off = __builtin_popcountll(todo);
     const int want = (n_off * slabs + part_stages - 1) / part_stages;
@@ -816,8 +828,8 @@ __device__ __forceinline__ void gms_rows_body(
   int gsel[C];
 
   // prologue: stage 0 goes straight to LDS
-  gidx[lane] = k_first >= 0 ? g_first : (in_range ? nbr[(size_t)k * n_dst + my_row] : -1);
-  int g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * n_dst + my_row] : -1;
+  gidx[lane] = k_first >= 0 ? g_first : (in_range ? nbr[(size_t)k * nbr_stride + my_row] : -1);
+  int g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * nbr_stride + my_row] : -1;
   wave_lds_fence();
   weights_issue(wreg, k, 0);
   if (active) gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
@@ -888,7 +900,7 @@ __device__ __forceinline__ void gms_rows_body(
     if (nk != k) {
       k_nxt = todo ? __builtin_ctzll(todo) : -1;
       if (todo) todo &= todo - 1;
-      g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * n_dst + my_row] : -1;
+      g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * nbr_stride + my_row] : -1;
     }
     __syncthreads();
     buf ^= 1;
@@ -910,7 +922,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
-    int c_src, int c_dst, int part_stages, SideJob side) {
+    int c_src, int c_dst, int part_stages, SideJob side, int pair_view) {
   // the leading workgroups of the grid run the side job, if there is one
   int block_x = blockIdx.x;
   if (side.blocks) {
@@ -921,7 +933,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     block_x -= side.blocks;
   }
   gms_rows_body<T, NT, S, RAW>(src, packed, dst, nbr, block_masks, perm, tile_order, n_dst, k_vol, c_src,
-                               c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z);
+                               c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z, pair_view);
 }
 
 // ---------------------------------------------------------------------------
@@ -1027,7 +1039,7 @@ bool raw_weights_enabled() {
 template <typename T, int NT, int S>
 int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
                 const unsigned long long *masks, const int32_t *perm, const int32_t *tile_order,
-                int tile_grid) {
+                int tile_grid, bool pair_view = false) {
   // With 64-column wave tiles the input gradient and the fp16 forward pass read the weight
   // tensor as it is (16-byte aligned rows of the tile) when the caller brings no re-laid
   // copy; the rest gets one, made here.  Measured: 64 -> 64 over 200k voxels, input gradient
@@ -1081,18 +1093,18 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   const int64_t slots = (int64_t)num_cus() * (NT == 4 ? 2 : 3);
   int part_stages = 0;
   unsigned gz = 1;
-  if ((int64_t)gx * gy * 2 <= slots && a.k_vol * slabs >= 8) {
+  if (!pair_view && (int64_t)gx * gy * 2 <= slots && a.k_vol * slabs >= 8) {
     part_stages = (a.k_vol * slabs + 1) / 2;
     gz = 2;
   }
   {
-    ProfileScope prof(raw == 4   ? "gms_rows_kernel(dgrad, bf16x3)"
+    ProfileScope prof(pair_view ? (a.transpose_w ? "gms_rows_kernel(dgrad, pair view)" : "gms_rows_kernel(fwd, pair view)") :raw == 4   ? "gms_rows_kernel(dgrad, bf16x3)"
                       : raw == 3 ? "gms_rows_kernel(fwd, bf16x3)"
                       : a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)",
                       a.stream);
     kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
-        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side);
+        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side, pair_view ? 1 : 0);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -1356,6 +1368,35 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p) {
     });
   return dispatch_rows_shape<float>(s, [&](auto nt, auto sv) {
     return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm, tile_order, tile_grid);
+  });
+}
+
+bool pair_view_gms_supported(const GmsArgs &a, const Plan *p) {
+  if (!p || !p->pv_in || a.dense_k >= 0 || a.k_vol != p->k_vol) return false;
+  if (a.transpose_w ? (a.n_dst != p->n_in || a.n_src != p->n_out) : (a.n_dst != p->n_out || a.n_src != p->n_in))
+    return false;
+  if (reinterpret_cast<uintptr_t>(a.dst) % 16) return false;
+  return shape_of(a).ok;
+}
+
+int launch_pair_view_gms(const GmsArgs &a, const Plan *p) {
+  if (!pair_view_gms_supported(a, p)) {
+    set_error("launch_pair_view_gms: unsupported shape or plan");
+    return FGMS_E_INVALID;
+  }
+  // the virtual rows stand in for the destination rows: tiles, the in-range test and the
+  // choice of the wave tile's width go by their number
+  GmsArgs v = a;
+  v.n_dst = p->pv_rows;
+  const Shape s = shape_of(v);
+  const int32_t *nbr = a.transpose_w ? p->pv_out : p->pv_in;
+  const int32_t *dest = a.transpose_w ? p->pv_in : p->pv_out;
+  if (a.dtype == FGMS_F16)
+    return dispatch_rows_shape<__half>(s, [&](auto nt, auto sv) {
+      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(v, s, nbr, p->pv_mask, dest, nullptr, 0, true);
+    });
+  return dispatch_rows_shape<float>(s, [&](auto nt, auto sv) {
+    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(v, s, nbr, p->pv_mask, dest, nullptr, 0, true);
   });
 }
 

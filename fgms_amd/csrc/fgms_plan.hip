@@ -52,6 +52,42 @@ __global__ void build_tables_kernel(const int32_t *__restrict__ kpos,
   if (atomicCAS(&nbr_in[(size_t)k * n_in + i], -1, o) != -1) flags[2] = 1;
 }
 
+// Pair view: the pair lists with every offset's run padded to a multiple of 64 rows
+// (pv_in / pv_out pre-filled with -1, pv_mask with 0).  Pair j of offset k goes to row
+// vpos[k] + j - kpos[k], vpos = the running sum of the padded run lengths.
+__global__ void pair_view_kernel(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+                                 const int32_t *__restrict__ omap, int k_vol, int n_pairs,
+                                 long long pv_rows, int32_t *__restrict__ pv_in,
+                                 int32_t *__restrict__ pv_out,
+                                 unsigned long long *__restrict__ pv_mask) {
+  __shared__ int kp[65];
+  __shared__ long long vp[65];
+  if ((int)threadIdx.x <= k_vol) kp[threadIdx.x] = kpos[threadIdx.x];
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    long long v = 0;
+    for (int k = 0; k < k_vol; ++k) {
+      vp[k] = v;
+      const int n = kp[k + 1] - kp[k];
+      if (n > 0) v += (n + 63) / 64 * 64;
+    }
+    vp[k_vol] = v;
+  }
+  __syncthreads();
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= kp[k_vol] || j >= n_pairs) return;
+  int lo = 0, hi = k_vol;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (kp[mid] <= j) lo = mid; else hi = mid;
+  }
+  const long long r = vp[lo] + (j - kp[lo]);
+  if (j < kp[lo] || r < 0 || r >= pv_rows) return;     // (a kpos that does not ascend)
+  pv_in[r] = imap[j];
+  pv_out[r] = omap[j];
+  if ((r & 63) == 0) pv_mask[r >> 6] = 1ull << lo;
+}
+
 // One wave per block of 64 consecutive rows: which offsets have a neighbour there.
 __global__ void block_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, int k_vol,
                                    unsigned long long *__restrict__ masks64) {
@@ -292,6 +328,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->band_count = 0; p->band_start = nullptr; p->band_cells = nullptr; p->bands_ok = false;
   p->tile_out = p->tile_in = nullptr; p->tile_grid_out = p->tile_grid_in = 0;
   p->fwd_ok = p->dgrad_ok = false;
+  p->pv_in = p->pv_out = nullptr; p->pv_mask = nullptr; p->pv_rows = 0;
   p->last_stream = s;
   int *flags = nullptr;
   int rc = FGMS_OK;
@@ -437,6 +474,32 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
+  // The pair view is built with the rest (before the one synchronisation) and kept only
+  // for maps sparse enough for a caller's layer to prefer it (see below).
+  static const bool pair_view = !(getenv("FGMS_PAIR_VIEW") && atoi(getenv("FGMS_PAIR_VIEW")) == 0);
+  if (pair_view && k_vol <= 64 && n_pairs > 0) {
+    p->pv_rows = (n_pairs + 64 * (int64_t)k_vol + 255) / 256 * 256;
+    if (pool_alloc((void **)&p->pv_in, (size_t)p->pv_rows * sizeof(int32_t), s) != FGMS_OK ||
+        pool_alloc((void **)&p->pv_out, (size_t)p->pv_rows * sizeof(int32_t), s) != FGMS_OK ||
+        pool_alloc((void **)&p->pv_mask, (size_t)(p->pv_rows / 64) * sizeof(unsigned long long), s) != FGMS_OK) {
+      free_tmp();
+      set_error("fgms_plan_create: pair view allocation failed");
+      return fail(FGMS_E_NOMEM);
+    }
+    if ((rc = fill_i32(p->pv_in, (size_t)p->pv_rows, -1, s)) || (rc = fill_i32(p->pv_out, (size_t)p->pv_rows, -1, s)) ||
+        (rc = fill_i32((int32_t *)p->pv_mask, (size_t)(p->pv_rows / 64) * 2, 0, s))) {
+      free_tmp();
+      return fail(rc);
+    }
+    pair_view_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(kpos, in_map, out_map, k_vol, (int)n_pairs,
+                                                                      (long long)p->pv_rows, p->pv_in, p->pv_out,
+                                                                      p->pv_mask);
+    if (hipGetLastError() != hipSuccess) {
+      free_tmp();
+      set_error("fgms_plan_create: pair view launch failed");
+      return fail(FGMS_E_HIP);
+    }
+  }
   int h[6] = {0, 0, 0, 0, 0, 0};
   if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
       hipStreamSynchronize(s) != hipSuccess) {
@@ -457,6 +520,14 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->bands_ok = !h[3];
   p->stages_out = h[4];
   p->stages_in = h[5];
+  // Dense maps never take the pair view (the widest layer, 256 fp16 channels, prefers it from
+  // about 2.2 row slots per pair on): drop it below 1.5 in both directions.
+  if (p->pv_in && kernel_policy() != 5 && (double)(p->stages_out > p->stages_in ? p->stages_out : p->stages_in) * 64.0 < 1.5 * (double)n_pairs) {
+    pool_free(p->pv_in, s, true);
+    pool_free(p->pv_out, s, true);
+    pool_free(p->pv_mask, s, true);
+    p->pv_in = p->pv_out = nullptr; p->pv_mask = nullptr; p->pv_rows = 0;
+  }
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
 }
@@ -474,6 +545,9 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->band_cells) pool_free(p->band_cells, p->last_stream, false);
   if (p->tile_out) pool_free(p->tile_out, p->last_stream, false);
   if (p->tile_in) pool_free(p->tile_in, p->last_stream, false);
+  if (p->pv_in) pool_free(p->pv_in, p->last_stream, false);
+  if (p->pv_out) pool_free(p->pv_out, p->last_stream, false);
+  if (p->pv_mask) pool_free(p->pv_mask, p->last_stream, false);
   delete p;
 }
 

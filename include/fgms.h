@@ -148,7 +148,11 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
  * output-stationary one can run: forward and input-gradient results are then the
  * same bit for bit from run to run (automatic dispatch gives wide layers over
  * scattered clouds, with few pairs per 64-row block and offset, to the
- * pair-stationary kernel, whose atomic sums depend on their order).
+ * pair-stationary kernel, whose atomic sums depend on their order; fp32 layers of
+ * that kind run the output-stationary kernel's body over the plan's pair view, also
+ * with atomic sums),
+ * 5 = forward and input gradient over the plan's pair view whenever the plan has
+ * one (plans created under this policy keep it for dense maps too).
  * Process-wide. */
 void fgms_set_kernel_policy(int policy);
 

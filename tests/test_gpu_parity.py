@@ -237,6 +237,40 @@ def test_baseline_configs_scaled(capi, oracle, cfg, variant):
     check_all(capi, oracle, L, policy=0, use_plan=False)
 
 
+@pytest.mark.parametrize("arch80", [False, True], ids=["", "tf32-mode"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("shape", [(32, 32), (64, 64), (128, 128), (64, 128), (256, 256), (96, 32)], ids=lambda s: "%dx%d" % s)
+def test_pair_view(capi, oracle, shape, dtype, arch80):
+    """Policy 5: forward and input gradient run the output-stationary kernel over the plan's
+    pair view (pair lists padded per offset to whole 64-row blocks, atomic sums); dense
+    submanifold map, strided map and a map with empty offsets."""
+    if arch80 and dtype == np.float16:
+        pytest.skip("the flag only concerns fp32 tensors")
+    capi.set_kernel_policy(5)
+    try:
+        L = layer(14, shape[0], shape[1], dtype)
+        D = G.to_dev(L)
+        plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+        capi.profile_reset()
+        capi.profile_enable(True)
+        G.run_fwd(capi, D, fused=True, arch80=arch80, plan=plan)
+        G.run_bwd(capi, D, plan=plan, arch80=arch80)
+        torch.cuda.synchronize()
+        capi.profile_enable(False)
+        names = [n for n, _ in capi.profile_records()]
+        capi.profile_reset()
+        plan.close()
+        assert any("pair view" in n and "fwd" in n for n in names), names
+        assert any("pair view" in n and "dgrad" in n for n in names), names
+        check_all(capi, oracle, L, policy=5, use_plan=True, arch80=arch80)
+        if shape == (64, 128):
+            check_all(capi, oracle, clouds.config_case(4, None, scale=0.08), policy=5, use_plan=True)
+            check_all(capi, oracle, clouds.config_case(4, "up", scale=0.08), policy=5, use_plan=True)
+            check_all(capi, oracle, clouds.config_case(3, None, scale=0.05), policy=5, use_plan=True)
+    finally:
+        capi.set_kernel_policy(0)
+
+
 @pytest.mark.parametrize("dtype", ["wide", "wide-fp32"], ids=["fp16", "fp32"])
 def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dtype):
     """A 256 -> 256 layer over a scattered cloud (few pairs per 64-row block and offset):
@@ -255,7 +289,9 @@ def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dty
     names = [n for n, _ in capi.profile_records()]
     capi.profile_reset()
     plan.close()
-    assert "gms_pairs_kernel(fwd)" in names and "gms_rows_kernel(fwd)" not in names, names
+    # (fp32: the output-stationary kernel's body over the plan's pair view, also with atomics)
+    want = "gms_pairs_kernel(fwd)" if dtype == "wide" else "gms_rows_kernel(fwd, pair view)"
+    assert want in names and "gms_rows_kernel(fwd)" not in names, names
     ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
     G.assert_close(out, ref, G.mode_of(L["in_feats"].dtype, False), "fwd")
 
