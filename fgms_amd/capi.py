@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfgms_hip.so")
 F32, F16 = 0, 1
 SYMBOLS = [
     "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_destroy",
-    "fgms_plan_usable", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
+    "fgms_plan_usable", "fgms_plan_stats", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
     "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map",
 ]
@@ -42,6 +42,8 @@ def lib():
     L.fgms_plan_destroy.argtypes = [vp]
     L.fgms_plan_destroy.restype = None
     L.fgms_plan_usable.argtypes = [vp, i32]
+    L.fgms_plan_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_int64)]
+    L.fgms_plan_stats.restype = i32
     L.fgms_fusion_fwd.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32,
                                   i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_fwd.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32,
@@ -143,6 +145,13 @@ class Plan:
 
     def usable(self, for_dgrad=False):
         return bool(lib().fgms_plan_usable(self._h, int(for_dgrad)))
+
+    def stats(self):
+        """dict(pairs, blocks_fwd, blocks_dgrad, pair_view_rows) as counted by the build; the
+        output-stationary kernels run 64 row slots per (64-row block, offset) in use."""
+        out = (ctypes.c_int64 * 4)()
+        _check(lib().fgms_plan_stats(self._h, out))
+        return {"pairs": out[0], "blocks_fwd": out[1], "blocks_dgrad": out[2], "pair_view_rows": out[3]}
 
     def close(self):
         if self._h:

@@ -247,20 +247,25 @@ int check_common(const void *a, const void *b, const void *c, const int32_t *kpo
 }
 
 // The output-stationary kernel multiplies every (64-row block, offset) combination in
-// use, 64 row slots each, whether or not a row has a pair there; the pair-stationary one
-// multiplies pairs only and pays with an atomic per result element.  Measured on MI355X
-// the atomics cost about as much as 240 (fp16) / 64 (fp32) channels of contraction per
-// pair, so the pair-stationary kernel wins when
-//   c_src + that  <  c_src * slots / pairs        (with 15 % in favour of the kernel
-// without atomics, whose results do not depend on the run).  Of the usual layers only wide
-// ones over scattered clouds qualify (256 -> 256 over a 50 k subsample: slots / pairs 2.6).
+// use, 64 row slots each, whether or not a row has a pair there; the pair-stationary
+// kernels multiply pairs only and pay with an atomic per result element.  Which one wins
+// depends on the row slots per pair of the map (1.0 .. 1.2 for surface-like clouds at full
+// density, 2 .. 3 for random subsamples of them) and on the channel count.  Measured on
+// MI355X over subsamples of a 200 k-voxel indoor-like cloud (35 k .. 200 k voxels, 32 .. 256
+// channels), the slots per pair at which both take the same time:
+//   fp32: 2.35 / 1.76 / 1.3 at 32 / 64 / 128 channels, i.e. about 1 + 45 / c (the MFMA time
+//         of the empty slots against a fixed cost per atomic);
+//   fp16: 2.25 .. 2.5 at every channel count (2.2 + 16 / c).
+// The kernel without atomics, whose results do not depend on the run, gets 5 % on top.
 bool sparse_rows(const GmsArgs &a, const Plan *plan) {
   const int stages = a.transpose_w ? plan->stages_in : plan->stages_out;
   if (stages <= 0 || plan->n_pairs <= 0) return false;   // (the plan's own pair count: a.n_pairs is a bound)
   const double slots_per_pair = (double)stages * 64.0 / (double)plan->n_pairs;
   const double c_src = a.transpose_w ? a.c_out : a.c_in;
-  const double atomics = a.dtype == FGMS_F16 ? 240.0 : 64.0;
-  return (c_src + atomics) * 1.15 < c_src * slots_per_pair;
+  const double even = a.dtype == FGMS_F16 ? 2.2 + 16.0 / c_src : 1.0 + 45.0 / c_src;
+  // (no break-even point was measured below 1.3: denser maps stay output-stationary)
+  const double need = 1.05 * even;
+  return slots_per_pair > (need > 1.4 ? need : 1.4);
 }
 
 enum class Route { kSkinny, kRows, kPairView, kPairs, kGeneric };
@@ -275,12 +280,13 @@ Route route_of(const GmsArgs &a, const Plan *plan) {
   if (!dense && g_policy != 2 && planned_gms_supported(a, plan) &&
       !(g_policy != 4 && sparse_rows(a, plan) && mfma_gms_supported(a)))
     return Route::kRows;
-  // Sparse maps, fp32: the output-stationary kernel's body over the plan's pair view (it streams
-  // the weights of a stage through LDS where the pair-stationary kernel holds a column block's
-  // weights of one offset, and gathers a row once per 64 columns either way).  Measured on
-  // 256 -> 256 over a 50 k-voxel scattered cloud: 245 us against 341 us fp32; fp16 96.6 against
-  // 96.3 us, which stays on the pair-stationary kernel.
-  if (g_policy == 0 && pair_view && a.dtype == FGMS_F32) return Route::kPairView;
+  // Which pair-stationary kernel: the output-stationary kernel's body over the plan's pair
+  // view streams the weights of a stage through LDS where gms_pairs_kernel holds a column
+  // block's weights of one offset.  Measured (same clouds): fp32 a tie up to 128 channels,
+  // 245 against 341 us at 256 -> 256 over 50 k voxels; fp16 14.2 against 18.3 us at 64
+  // channels over 35 k voxels, a tie from 128 channels on (96.6 against 96.3 us at 256).
+  if (g_policy == 0 && pair_view && (a.dtype == FGMS_F32 || (a.transpose_w ? a.c_out : a.c_in) <= 64))
+    return Route::kPairView;
   return mfma_gms_supported(a) ? Route::kPairs : Route::kGeneric;
 }
 

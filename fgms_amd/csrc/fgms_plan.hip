@@ -520,9 +520,9 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->bands_ok = !h[3];
   p->stages_out = h[4];
   p->stages_in = h[5];
-  // Dense maps never take the pair view (the widest layer, 256 fp16 channels, prefers it from
-  // about 2.2 row slots per pair on): drop it below 1.5 in both directions.
-  if (p->pv_in && kernel_policy() != 5 && (double)(p->stages_out > p->stages_in ? p->stages_out : p->stages_in) * 64.0 < 1.5 * (double)n_pairs) {
+  // Dense maps never take the pair view (fp32 layers prefer it from about 1 + 45 / channels
+  // row slots per pair on, never below 1.4): drop it below 1.35 in both directions.
+  if (p->pv_in && kernel_policy() != 5 && (double)(p->stages_out > p->stages_in ? p->stages_out : p->stages_in) * 64.0 < 1.35 * (double)n_pairs) {
     pool_free(p->pv_in, s, true);
     pool_free(p->pv_out, s, true);
     pool_free(p->pv_mask, s, true);
@@ -555,6 +555,19 @@ int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad) {
   const Plan *p = (const Plan *)plan;
   if (!p) return 0;
   return for_dgrad ? (p->dgrad_ok ? 1 : 0) : (p->fwd_ok ? 1 : 0);
+}
+
+int fgms_plan_stats(const fgms_plan_t *plan, int64_t stats[4]) {
+  const Plan *p = (const Plan *)plan;
+  if (!p || !stats) {
+    set_error("fgms_plan_stats: null argument");
+    return FGMS_E_INVALID;
+  }
+  stats[0] = p->n_pairs;
+  stats[1] = p->stages_out;
+  stats[2] = p->stages_in;
+  stats[3] = p->pv_in ? p->pv_rows : 0;
+  return FGMS_OK;
 }
 
 }  // extern "C"

@@ -76,6 +76,12 @@ int fgms_plan_create(fgms_plan_t **plan, const int32_t *kpos,
 void fgms_plan_destroy(fgms_plan_t *plan);
 /* 1 if the output-stationary kernels can use it for forward / for dgrad. */
 int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad);
+/* What the build counted (no counterpart in the reference): stats[0] = pairs in the map,
+ * stats[1] / stats[2] = (64-row block, offset) combinations with at least one pair in the
+ * forward / input-gradient direction (the output-stationary kernels run 64 row slots for
+ * each, so stats[1] * 64 / stats[0] is their row slots per pair), stats[3] = rows of the
+ * pair view (0: the plan keeps none).  Returns FGMS_OK or FGMS_E_INVALID. */
+int fgms_plan_stats(const fgms_plan_t *plan, int64_t stats[4]);
 
 /*
  * Replaces ConvolutionForwardFused  (backend/spconv.cu:23-246; pybind name
