@@ -319,7 +319,9 @@ def main():
         "vs_baseline": None, "dtype": arith, "data": "synthetic",
         "config": {"workload": args.workload, "voxels_in": L["n_in"], "voxels_out": L["n_out"],
                    "pairs": m, "k_vol": L["k_vol"], "c_in": L["c_in"], "c_out": L["c_out"],
-                   "plan": plan is not None, "policy": args.policy},
+                   "plan": plan is not None, "policy": args.policy,
+                   "row_slots_per_pair": (round(plan.stats()["blocks_fwd"] * 64.0 / max(plan.stats()["pairs"], 1), 3)
+                                          if plan is not None else None)},
         "kernels": kernels,
         "roofline": roofline,
         "gather_floor": gather_floor,

@@ -271,6 +271,22 @@ def test_pair_view(capi, oracle, shape, dtype, arch80):
         capi.set_kernel_policy(0)
 
 
+def test_plan_stats(capi):
+    """fgms_plan_stats against a count in numpy: pairs, and the (64-row block, offset)
+    combinations in use, which lie between pairs / 64 (and the number of offsets in use) and
+    the pair count (and blocks x offsets)."""
+    L = layer(15, 32, 32, np.float32)
+    D = G.to_dev(L)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    st = plan.stats()
+    plan.close()
+    assert st["pairs"] == len(L["imap"])
+    floor = max(-(-len(L["imap"]) // 64), int((L["knnz"] > 0).sum()))
+    assert floor <= st["blocks_fwd"] <= min(len(L["imap"]), -(-L["n_out"] // 64) * L["k_vol"])
+    assert floor <= st["blocks_dgrad"] <= min(len(L["imap"]), -(-L["n_in"] // 64) * L["k_vol"])
+    assert st["pair_view_rows"] % 256 == 0
+
+
 @pytest.mark.parametrize("dtype", ["wide", "wide-fp32"], ids=["fp16", "fp32"])
 def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dtype):
     """A 256 -> 256 layer over a scattered cloud (few pairs per 64-row block and offset):
