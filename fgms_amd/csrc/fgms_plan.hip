@@ -8,6 +8,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <map>
+#include <mutex>
 #include <vector>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -257,18 +259,31 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restr
 // the other cells of its XCD (a few hundred).
 __global__ void band_cells_kernel(const int32_t *__restrict__ band_start, int k_vol, int bands,
                                   int32_t *__restrict__ cells) {
+  // the pair counts of the XCD's cells (and which of its bands a cell lies in) go to LDS
+  // once: every thread compares with all of them, and the integer divisions of the cell
+  // arithmetic would otherwise dominate the loop
+  constexpr int kCached = 2048;
+  __shared__ int count[kCached];
+  __shared__ short band_of[kCached];
   const int per_xcd = (bands / 8) * k_vol;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;   // cell number inside its XCD: (band / 8) * k_vol + k
-  const int x = blockIdx.y, group = 1 << blockIdx.z;
-  if (c >= per_xcd) return;
+  const int x = blockIdx.y, shift = blockIdx.z;           // groups of 1 << shift bands
   auto pairs_of = [&](int cell) {
     const int k = cell % k_vol, band = (cell / k_vol) * 8 + x;
     return band_start[k * (bands + 1) + band + 1] - band_start[k * (bands + 1) + band];
   };
-  const int mine = pairs_of(c), my_group = (c / k_vol) / group;
+  for (int o = threadIdx.x; o < per_xcd && o < kCached; o += blockDim.x) {
+    count[o] = pairs_of(o);
+    band_of[o] = (short)(o / k_vol);
+  }
+  __syncthreads();
+  if (c >= per_xcd) return;
+  const int mine = pairs_of(c), my_group = (c / k_vol) >> shift;
   int rank = 0;
   for (int o = 0; o < per_xcd; ++o) {
-    const int theirs = pairs_of(o), their_group = (o / k_vol) / group;
+    const bool cached = o < kCached;
+    const int theirs = cached ? count[o] : pairs_of(o);
+    const int their_group = (cached ? (int)band_of[o] : o / k_vol) >> shift;
     const bool before = their_group != my_group ? their_group < my_group
                                                  : (theirs > mine || (theirs == mine && o < c));
     rank += before ? 1 : 0;
@@ -287,7 +302,25 @@ __global__ void permute_table_kernel(const int32_t *__restrict__ in, const int32
   const int pos = blockIdx.x * blockDim.x + threadIdx.x;
   if (pos >= n_rows) return;
   const int row = perm[pos];
-  for (int k = 0; k < k_vol; ++k) out[(size_t)k * n_rows + pos] = in[(size_t)k * n_rows + row];
+  // (one offset per blockIdx.y: 27 independent loads per row in flight instead of a loop)
+  for (int k = blockIdx.y; k < k_vol; k += gridDim.y) out[(size_t)k * n_rows + pos] = in[(size_t)k * n_rows + row];
+}
+
+// The two directions of a plan (output side, input side) are chains of a dozen small
+// launches each (masks, radix sort, permutation, block masks, tile order) that do not
+// depend on each other; at 200 k rows every launch is bound by its latency, so the input
+// side's chain runs on a stream of the library's own (default priority, one per device,
+// created on first use) next to the caller's.  nullptr: creation failed, one stream is used.
+hipStream_t side_stream(int device) {
+  static std::mutex m;
+  static std::map<int, hipStream_t> streams;
+  std::lock_guard<std::mutex> lock(m);
+  auto it = streams.find(device);
+  if (it != streams.end()) return it->second;
+  hipStream_t st = nullptr;
+  if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) st = nullptr;
+  streams[device] = st;
+  return st;
 }
 
 int fill_i32(int32_t *p, size_t n, int32_t v, hipStream_t s) {
@@ -377,6 +410,20 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
+  // fork: the input side's chain waits for the tables only
+  static const bool two_streams = !(getenv("FGMS_PLAN_STREAMS") && atoi(getenv("FGMS_PLAN_STREAMS")) == 1);
+  hipStream_t s2 = (two_streams && k_vol <= 64 && n_in > 0 && n_out > 0) ? side_stream(p->device) : nullptr;
+  hipEvent_t forked = nullptr, joined = nullptr;
+  if (s2) {
+    if (hipEventCreateWithFlags(&forked, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&joined, hipEventDisableTiming) != hipSuccess ||
+        hipEventRecord(forked, s) != hipSuccess || hipStreamWaitEvent(s2, forked, 0) != hipSuccess) {
+      if (forked) (void)hipEventDestroy(forked);
+      if (joined) (void)hipEventDestroy(joined);
+      forked = joined = nullptr;
+      s2 = nullptr;      // (nothing was queued on it)
+    }
+  }
   band_bounds_kernel<<<(unsigned)k_vol, 128, 0, s>>>(kpos, out_map, (int)n_pairs, p->band_count,
                                                      band_rows > 0 ? band_rows : 1, p->band_start);
   {
@@ -391,6 +438,15 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   unsigned long long *tmp_mask[2] = {nullptr, nullptr};
   std::vector<void *> tmp_more;
   auto free_tmp = [&]() {
+    if (s2 && !synced) {
+      // work of the side stream may still use the temporaries: drain both streams first
+      (void)hipStreamSynchronize(s2);
+      (void)hipStreamSynchronize(s);
+      synced = true;
+    }
+    if (forked) (void)hipEventDestroy(forked);
+    if (joined) (void)hipEventDestroy(joined);
+    forked = joined = nullptr;
     for (int d = 0; d < 2; ++d) {
       if (tmp_tab[d]) pool_free(tmp_tab[d], s, synced);
       if (tmp_mask[d]) pool_free(tmp_mask[d], s, synced);
@@ -403,6 +459,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   if (k_vol <= 64) {
     for (int d = 0; d < 2; ++d) {
       const int64_t n = d ? n_in : n_out;
+      hipStream_t sd = (d == 1 && s2) ? s2 : s;   // the stream of this direction's chain
       const size_t blocks = d ? bi : bo;
       int32_t *&tab = d ? p->nbr_in : p->nbr_out;
       int32_t *&perm = d ? p->perm_in : p->perm_out;
@@ -410,32 +467,32 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       if (n == 0) continue;
       if (sort_rows && n > 64) {
         int32_t *sorted = nullptr;
-        if (pool_alloc((void **)&tmp_mask[d], (size_t)n * sizeof(unsigned long long), s) != FGMS_OK ||
-            pool_alloc((void **)&perm, (size_t)n * sizeof(int32_t), s) != FGMS_OK ||
-            pool_alloc((void **)&sorted, (size_t)n * k_vol * sizeof(int32_t), s) != FGMS_OK) {
+        if (pool_alloc((void **)&tmp_mask[d], (size_t)n * sizeof(unsigned long long), sd) != FGMS_OK ||
+            pool_alloc((void **)&perm, (size_t)n * sizeof(int32_t), sd) != FGMS_OK ||
+            pool_alloc((void **)&sorted, (size_t)n * k_vol * sizeof(int32_t), sd) != FGMS_OK) {
           if (sorted) pool_free(sorted, s, synced);
           free_tmp();
           set_error("fgms_plan_create: reorder allocation failed");
           return fail(FGMS_E_NOMEM);
         }
-        row_masks_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(tab, (int)n, k_vol, tmp_mask[d]);
+        row_masks_kernel<<<(unsigned)((n + 255) / 256), 256, 0, sd>>>(tab, (int)n, k_vol, tmp_mask[d]);
         // stable LSD radix sort over the k_vol significant bits of the masks
         unsigned long long *keys_out = nullptr;
         int32_t *rows_in = nullptr;
         void *sort_tmp = nullptr;
         size_t sort_bytes = 0;
-        bool ok = pool_alloc((void **)&keys_out, (size_t)n * sizeof(unsigned long long), s) == FGMS_OK;
+        bool ok = pool_alloc((void **)&keys_out, (size_t)n * sizeof(unsigned long long), sd) == FGMS_OK;
         if (ok) tmp_more.push_back(keys_out);
-        ok = ok && pool_alloc((void **)&rows_in, (size_t)n * sizeof(int32_t), s) == FGMS_OK;
+        ok = ok && pool_alloc((void **)&rows_in, (size_t)n * sizeof(int32_t), sd) == FGMS_OK;
         if (ok) tmp_more.push_back(rows_in);
         ok = ok && rocprim::radix_sort_pairs(nullptr, sort_bytes, tmp_mask[d], keys_out, rows_in, perm,
-                                             (size_t)n, 0u, (unsigned)k_vol, s) == hipSuccess;
-        ok = ok && pool_alloc(&sort_tmp, sort_bytes, s) == FGMS_OK;
+                                             (size_t)n, 0u, (unsigned)k_vol, sd) == hipSuccess;
+        ok = ok && pool_alloc(&sort_tmp, sort_bytes, sd) == FGMS_OK;
         if (ok) tmp_more.push_back(sort_tmp);
         if (ok) {
-          iota_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(rows_in, (int)n);
+          iota_kernel<<<(unsigned)((n + 255) / 256), 256, 0, sd>>>(rows_in, (int)n);
           ok = rocprim::radix_sort_pairs(sort_tmp, sort_bytes, tmp_mask[d], keys_out, rows_in, perm,
-                                         (size_t)n, 0u, (unsigned)k_vol, s) == hipSuccess;
+                                         (size_t)n, 0u, (unsigned)k_vol, sd) == hipSuccess;
         }
         if (!ok) {
           pool_free(sorted, s, synced);
@@ -443,60 +500,39 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
           set_error("fgms_plan_create: row sort failed");
           return fail(FGMS_E_HIP);
         }
-        permute_table_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(tab, perm, (int)n, k_vol, sorted);
+        permute_table_kernel<<<dim3((unsigned)((n + 255) / 256), (unsigned)k_vol), 256, 0, sd>>>(tab, perm, (int)n, k_vol, sorted);
         tmp_tab[d] = tab;      // the unsorted table, freed after the sync
         tab = sorted;
       }
-      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, s>>>(tab, (int)n, k_vol, mask);
-      count_stages_kernel<<<1, 1024, 0, s>>>(mask, (int)blocks, flags + 4 + d);
+      block_masks_kernel<<<(unsigned)((blocks + 3) / 4), 256, 0, sd>>>(tab, (int)n, k_vol, mask);
+      count_stages_kernel<<<1, 1024, 0, sd>>>(mask, (int)blocks, flags + 4 + d);
       // tile -> XCD homes pay off once every XCD has a few dozen tiles of its own
       static const bool xcd_homes = !(getenv("FGMS_XCD_HOME") && atoi(getenv("FGMS_XCD_HOME")) == 0);
       const int n_tiles = (int)((n + 255) / 256);
       if (xcd_homes && n_tiles >= 256 && (size_t)n_tiles * sizeof(int32_t) <= 60000) {
         int32_t *&order = d ? p->tile_in : p->tile_out;
         const int cap = (n_tiles + 7) / 8;
-        if (pool_alloc((void **)&order, (size_t)cap * 8 * sizeof(int32_t), s) != FGMS_OK) {
+        if (pool_alloc((void **)&order, (size_t)cap * 8 * sizeof(int32_t), sd) != FGMS_OK) {
           free_tmp();
           return fail(FGMS_E_NOMEM);
         }
         (d ? p->tile_grid_in : p->tile_grid_out) = cap * 8;
-        if ((rc = fill_i32(order, (size_t)cap * 8, -1, s))) {
+        if ((rc = fill_i32(order, (size_t)cap * 8, -1, sd))) {
           free_tmp();
           return fail(rc);
         }
-        tile_order_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), s>>>(
+        tile_order_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), sd>>>(
             perm, mask, (int)n, n_tiles, cap, num_cus() >= 8 ? num_cus() / 8 : 1, order);
       }
+    }
+    if (s2 && (hipEventRecord(joined, s2) != hipSuccess || hipStreamWaitEvent(s, joined, 0) != hipSuccess)) {
+      free_tmp();
+      set_error("fgms_plan_create: joining the side stream failed");
+      return fail(FGMS_E_HIP);
     }
     if (hipGetLastError() != hipSuccess) {
       free_tmp();
       set_error("fgms_plan_create: reorder / mask build launch failed");
-      return fail(FGMS_E_HIP);
-    }
-  }
-  // The pair view is built with the rest (before the one synchronisation) and kept only
-  // for maps sparse enough for a caller's layer to prefer it (see below).
-  static const bool pair_view = !(getenv("FGMS_PAIR_VIEW") && atoi(getenv("FGMS_PAIR_VIEW")) == 0);
-  if (pair_view && k_vol <= 64 && n_pairs > 0) {
-    p->pv_rows = (n_pairs + 64 * (int64_t)k_vol + 255) / 256 * 256;
-    if (pool_alloc((void **)&p->pv_in, (size_t)p->pv_rows * sizeof(int32_t), s) != FGMS_OK ||
-        pool_alloc((void **)&p->pv_out, (size_t)p->pv_rows * sizeof(int32_t), s) != FGMS_OK ||
-        pool_alloc((void **)&p->pv_mask, (size_t)(p->pv_rows / 64) * sizeof(unsigned long long), s) != FGMS_OK) {
-      free_tmp();
-      set_error("fgms_plan_create: pair view allocation failed");
-      return fail(FGMS_E_NOMEM);
-    }
-    if ((rc = fill_i32(p->pv_in, (size_t)p->pv_rows, -1, s)) || (rc = fill_i32(p->pv_out, (size_t)p->pv_rows, -1, s)) ||
-        (rc = fill_i32((int32_t *)p->pv_mask, (size_t)(p->pv_rows / 64) * 2, 0, s))) {
-      free_tmp();
-      return fail(rc);
-    }
-    pair_view_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(kpos, in_map, out_map, k_vol, (int)n_pairs,
-                                                                      (long long)p->pv_rows, p->pv_in, p->pv_out,
-                                                                      p->pv_mask);
-    if (hipGetLastError() != hipSuccess) {
-      free_tmp();
-      set_error("fgms_plan_create: pair view launch failed");
       return fail(FGMS_E_HIP);
     }
   }
@@ -520,13 +556,30 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->bands_ok = !h[3];
   p->stages_out = h[4];
   p->stages_in = h[5];
-  // Dense maps never take the pair view (fp32 layers prefer it from about 1 + 45 / channels
-  // row slots per pair on, never below 1.4): drop it below 1.35 in both directions.
-  if (p->pv_in && kernel_policy() != 5 && (double)(p->stages_out > p->stages_in ? p->stages_out : p->stages_in) * 64.0 < 1.35 * (double)n_pairs) {
-    pool_free(p->pv_in, s, true);
-    pool_free(p->pv_out, s, true);
-    pool_free(p->pv_mask, s, true);
-    p->pv_in = p->pv_out = nullptr; p->pv_mask = nullptr; p->pv_rows = 0;
+  // The pair view, for maps sparse enough that some layer would take it (fp32 layers prefer
+  // it from about 1 + 45 / channels row slots per pair on, never below 1.4): built after the
+  // counts are known, with a synchronisation of its own, so that dense maps pay nothing.
+  static const bool pair_view = !(getenv("FGMS_PAIR_VIEW") && atoi(getenv("FGMS_PAIR_VIEW")) == 0);
+  const int most = p->stages_out > p->stages_in ? p->stages_out : p->stages_in;
+  if (pair_view && k_vol <= 64 && n_pairs > 0 &&
+      (kernel_policy() == 5 || (double)most * 64.0 >= 1.35 * (double)n_pairs)) {
+    p->pv_rows = (n_pairs + 64 * (int64_t)k_vol + 255) / 256 * 256;
+    if (pool_alloc((void **)&p->pv_in, (size_t)p->pv_rows * sizeof(int32_t), s) != FGMS_OK ||
+        pool_alloc((void **)&p->pv_out, (size_t)p->pv_rows * sizeof(int32_t), s) != FGMS_OK ||
+        pool_alloc((void **)&p->pv_mask, (size_t)(p->pv_rows / 64) * sizeof(unsigned long long), s) != FGMS_OK) {
+      set_error("fgms_plan_create: pair view allocation failed");
+      return fail(FGMS_E_NOMEM);
+    }
+    if ((rc = fill_i32(p->pv_in, (size_t)p->pv_rows, -1, s)) || (rc = fill_i32(p->pv_out, (size_t)p->pv_rows, -1, s)) ||
+        (rc = fill_i32((int32_t *)p->pv_mask, (size_t)(p->pv_rows / 64) * 2, 0, s)))
+      return fail(rc);
+    pair_view_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(kpos, in_map, out_map, k_vol, (int)n_pairs,
+                                                                      (long long)p->pv_rows, p->pv_in, p->pv_out,
+                                                                      p->pv_mask);
+    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(s) != hipSuccess) {
+      set_error("fgms_plan_create: pair view build failed");
+      return fail(FGMS_E_HIP);
+    }
   }
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
