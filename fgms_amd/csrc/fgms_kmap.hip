@@ -16,6 +16,7 @@
 //   3. scan     exclusive prefix sum over the (offset, block) counts (rocPRIM)
 //   4. write    hits are compacted in (offset, row) order: block base from the
 //               scan, rank inside the block from wave ballots
+#include <stdlib.h>
 #include <string.h>
 
 #include <vector>
@@ -56,7 +57,14 @@ __global__ void kmap_fill_kernel(unsigned long long *__restrict__ keys, int32_t 
   }
 }
 
-// flags[0]: an input coordinate is outside the packable range
+__global__ void kmap_fill_none_kernel(int32_t *__restrict__ p, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = -1;
+}
+
+// flags[0]: an input coordinate is outside the packable range; flags[2]: two input rows share
+// their coordinates
 __global__ void kmap_insert_kernel(const int32_t *__restrict__ coords, int n,
                                    unsigned long long *__restrict__ keys, int32_t *__restrict__ vals,
                                    unsigned long long mask, int *__restrict__ flags) {
@@ -71,6 +79,7 @@ __global__ void kmap_insert_kernel(const int32_t *__restrict__ coords, int n,
   while (true) {                       // ends: load <= 0.5, a free or equal slot exists
     const unsigned long long prev = atomicCAS(&keys[slot], kEmptyKey, key);
     if (prev == kEmptyKey || prev == key) {
+      if (prev == key) flags[2] = 1;
       atomicMin(&vals[slot], i);
       return;
     }
@@ -80,11 +89,16 @@ __global__ void kmap_insert_kernel(const int32_t *__restrict__ coords, int n,
 
 // grid (blocks of 256 output rows, k_vol).  table[k][o] = input row or -1;
 // counts[k * n_blocks + block] = hits of the block.
+// mirror_k > 0 (= k_vol, odd): the map is its own mirror image -- one coordinate list on
+// both sides, unique coordinates, offsets[k_vol - 1 - k] = -offsets[k] -- so a hit (k, o) -> i
+// is also the hit (k_vol - 1 - k, i) -> o.  The grid then covers the offsets up to the centre
+// only and fills the other half of the table (pre-filled with -1) from its hits: half the
+// hash lookups.  kmap_count_kernel then counts that half's hits per block.
 __global__ __launch_bounds__(kBlock) void kmap_lookup_kernel(
     const int32_t *__restrict__ out_coords, int n_out, const int32_t *__restrict__ offsets,
     int stride, int skip_offset, const unsigned long long *__restrict__ keys,
     const int32_t *__restrict__ vals, unsigned long long mask, int32_t *__restrict__ table,
-    int32_t *__restrict__ counts) {
+    int32_t *__restrict__ counts, int mirror_k) {
   __shared__ int block_hits;
   const int k = blockIdx.y, o = blockIdx.x * kBlock + threadIdx.x;
   if (threadIdx.x == 0) block_hits = 0;
@@ -105,7 +119,26 @@ __global__ __launch_bounds__(kBlock) void kmap_lookup_kernel(
     }
   }
   if (o < n_out) table[(size_t)k * n_out + o] = hit;
+  if (mirror_k > 0 && hit >= 0 && 2 * k + 1 < mirror_k) {
+    const int km = mirror_k - 1 - k;
+    table[(size_t)km * n_out + hit] = o;      // (counted by kmap_count_kernel afterwards)
+  }
   const unsigned long long b = __ballot(hit >= 0);
+  if (threadIdx.x % 64 == 0 && b) atomicAdd(&block_hits, __builtin_popcountll(b));
+  __syncthreads();
+  if (threadIdx.x == 0) counts[(size_t)k * gridDim.x + blockIdx.x] = block_hits;
+}
+
+// grid (blocks of 256 output rows, offsets from k_first on): counts[k * n_blocks + block] =
+// entries >= 0 of the block.
+__global__ __launch_bounds__(kBlock) void kmap_count_kernel(const int32_t *__restrict__ table, int n_out,
+                                                            int k_first, int32_t *__restrict__ counts) {
+  __shared__ int block_hits;
+  const int k = k_first + blockIdx.y, o = blockIdx.x * kBlock + threadIdx.x;
+  if (threadIdx.x == 0) block_hits = 0;
+  __syncthreads();
+  const bool hit = o < n_out && table[(size_t)k * n_out + o] >= 0;
+  const unsigned long long b = __ballot(hit);
   if (threadIdx.x % 64 == 0 && b) atomicAdd(&block_hits, __builtin_popcountll(b));
   __syncthreads();
   if (threadIdx.x == 0) counts[(size_t)k * gridDim.x + blockIdx.x] = block_hits;
@@ -145,10 +178,21 @@ __global__ void kmap_finish_kernel(const int32_t *__restrict__ bases, int k_vol,
 
 }  // namespace
 
-int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
-                     const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
-                     int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,
-                     int32_t *kpos, int64_t *n_pairs, hipStream_t s) {
+namespace {
+int build_kernel_map_impl(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
+                          const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
+                          int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,
+                          int32_t *kpos, int64_t *n_pairs, hipStream_t s, bool allow_mirror, bool *retry) {
+  *retry = false;
+  // A submanifold map (one coordinate list on both sides, symmetric offsets) is its own
+  // mirror image: half of the lookups give the other half (see kmap_lookup_kernel).
+  // FGMS_KMAP_MIRROR=0 looks every offset up.
+  static const bool mirror_on = !(getenv("FGMS_KMAP_MIRROR") && atoi(getenv("FGMS_KMAP_MIRROR")) == 0);
+  bool mirror = allow_mirror && mirror_on && in_coords == out_coords && n_in == n_out && stride == 1 &&
+                k_vol >= 3 && k_vol % 2 == 1 && (skip_offset < 0 || skip_offset == k_vol / 2);
+  for (int k = 0; mirror && k < k_vol; ++k)
+    for (int c = 0; c < 3; ++c)
+      if (offsets_host[3 * (k_vol - 1 - k) + c] != -offsets_host[3 * k + c]) mirror = false;
   size_t slots = 64;
   while (slots < 2 * (size_t)n_in) slots <<= 1;
   const int n_blocks = (int)((n_out + kBlock - 1) / kBlock);
@@ -203,8 +247,17 @@ int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_
   if (n_out > 0) {
     {
       ProfileScope prof("kmap_lookup_kernel", s);
-      kmap_lookup_kernel<<<dim3((unsigned)n_blocks, (unsigned)k_vol), kBlock, 0, s>>>(
-          out_coords, (int)n_out, offs, stride, skip_offset, keys, vals, mask, table, counts);
+      if (mirror) {
+        const size_t half = (size_t)(k_vol / 2) * n_out;     // the offsets after the centre
+        size_t blocks = (half + 1023) / 1024;
+        kmap_fill_none_kernel<<<(unsigned)(blocks > 65535 ? 65535 : blocks), 256, 0, s>>>(
+            table + (size_t)(k_vol / 2 + 1) * n_out, half);
+      }
+      kmap_lookup_kernel<<<dim3((unsigned)n_blocks, (unsigned)(mirror ? k_vol / 2 + 1 : k_vol)), kBlock, 0, s>>>(
+          out_coords, (int)n_out, offs, stride, skip_offset, keys, vals, mask, table, counts, mirror ? k_vol : 0);
+      if (mirror)
+        kmap_count_kernel<<<dim3((unsigned)n_blocks, (unsigned)(k_vol / 2)), kBlock, 0, s>>>(table, (int)n_out,
+                                                                                            k_vol / 2 + 1, counts);
     }
   }
   if (rocprim::exclusive_scan(scan_tmp, scan_bytes, counts, bases, 0, n_counts, rocprim::plus<int32_t>(), s) != hipSuccess)
@@ -216,12 +269,16 @@ int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_
   }
   kmap_finish_kernel<<<(unsigned)((k_vol + 1 + 255) / 256), 256, 0, s>>>(bases, k_vol, n_blocks, kernel_nnz, kpos, flags + 1);
   if (hipGetLastError() != hipSuccess) return fail("kernel launch failed");
-  int32_t h[2] = {0, 0};
+  int32_t h[3] = {0, 0, 0};
   if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
       hipStreamSynchronize(s) != hipSuccess)
     return fail("reading the result size failed");
   synced = true;
   release();
+  if (mirror && h[2] && !h[0]) {       // rows that share coordinates: every offset has to be looked up
+    *retry = true;
+    return FGMS_OK;
+  }
   if (h[0]) {
     set_error("fgms_build_kernel_map: an input coordinate is outside [-2^20, 2^20)");
     return FGMS_E_INVALID;
@@ -232,6 +289,20 @@ int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_
     return FGMS_E_INVALID;
   }
   return FGMS_OK;
+}
+}  // namespace
+
+int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
+                     const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
+                     int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,
+                     int32_t *kpos, int64_t *n_pairs, hipStream_t s) {
+  bool retry = false;
+  int rc = build_kernel_map_impl(in_coords, n_in, out_coords, n_out, offsets_host, k_vol, stride, skip_offset,
+                                 in_map, out_map, capacity, kernel_nnz, kpos, n_pairs, s, true, &retry);
+  if (rc == FGMS_OK && retry)
+    rc = build_kernel_map_impl(in_coords, n_in, out_coords, n_out, offsets_host, k_vol, stride, skip_offset,
+                               in_map, out_map, capacity, kernel_nnz, kpos, n_pairs, s, false, &retry);
+  return rc;
 }
 
 }  // namespace fgms

@@ -61,6 +61,29 @@ def test_duplicate_input_coordinates_take_the_smallest_row(capi):
     check(capi, twice, vox, clouds.offsets_cube(3))
 
 
+def check_one_list(capi, vox, offsets, skip=None):
+    """One device tensor on both sides: the builder may then take half of the lookups from the
+    other half (a submanifold map is its own mirror image)."""
+    want = clouds.build_kernel_map(vox, vox, offsets, 1, skip)
+    d = dev(vox)
+    got = capi.build_kernel_map(d, d, offsets, 1, skip)
+    for g, w, name in zip(got, want, ("in_map", "out_map", "kernel_nnz", "kpos")):
+        assert np.array_equal(g.cpu().numpy(), w), name
+    return got
+
+
+def test_one_coordinate_list_on_both_sides(capi):
+    vox = random_cloud(56)
+    check_one_list(capi, vox, clouds.offsets_cube(3))
+    check_one_list(capi, vox, clouds.offsets_cube(3), skip=13)
+    check_one_list(capi, random_cloud(57, shift=-25), clouds.offsets_cube(5))
+    check_one_list(capi, vox, clouds.offsets_cube(2))               # offsets without mirror images
+    check_one_list(capi, vox, clouds.offsets_cube(3)[::-1][[1, 0] + list(range(2, 27))])   # ... in an order that is not mirrored
+    check_one_list(capi, vox[:1], clouds.offsets_cube(3))
+    twice = np.concatenate([vox, vox[::3]])                          # rows that share coordinates: no mirroring
+    check_one_list(capi, twice, clouds.offsets_cube(3))
+
+
 def test_empty_sides(capi):
     vox = random_cloud(55, n=300)
     none = np.zeros((0, 3), np.int32)
@@ -87,6 +110,8 @@ def test_headline_cloud_full_size_and_feeds_the_kernels(capi, oracle):
     vox = clouds.indoor_cloud()
     imap, omap, knnz, kpos = check(capi, vox, vox, clouds.offsets_cube(3))
     assert imap.numel() == 2112390
+    for g, w in zip(check_one_list(capi, vox, clouds.offsets_cube(3)), (imap, omap, knnz, kpos)):
+        assert torch.equal(g, w)
     n = len(vox)
     x = torch.randn(n, 32, device="cuda").half()
     w = (torch.randn(27, 32, 32, device="cuda") * 0.05).half()
