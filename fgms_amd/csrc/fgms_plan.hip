@@ -280,6 +280,7 @@ __global__ void band_cells_kernel(const int32_t *__restrict__ band_start, int k_
   if (c >= per_xcd) return;
   const int mine = pairs_of(c), my_group = (c / k_vol) >> shift;
   int rank = 0;
+#pragma unroll 8      // (independent LDS reads in flight: the loop is bound by their latency)
   for (int o = 0; o < per_xcd; ++o) {
     const bool cached = o < kCached;
     const int theirs = cached ? count[o] : pairs_of(o);
