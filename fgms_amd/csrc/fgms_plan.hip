@@ -128,10 +128,12 @@ __global__ __launch_bounds__(1024) void count_stages_kernel(const unsigned long 
 }
 
 // rmask[row] = bit k set iff row has a neighbour through offset k.
+// Also rows[row] = row, the values the sort permutes.
 __global__ void row_masks_kernel(const int32_t *__restrict__ nbr, int n_rows, int k_vol,
-                                 unsigned long long *__restrict__ rmask) {
+                                 unsigned long long *__restrict__ rmask, int32_t *__restrict__ rows) {
   const int row = blockIdx.x * blockDim.x + threadIdx.x;
   if (row >= n_rows) return;
+  rows[row] = row;
   unsigned long long m = 0;
   for (int k = 0; k < k_vol; ++k)
     if (nbr[(size_t)k * n_rows + row] >= 0) m |= 1ull << k;
@@ -177,7 +179,7 @@ __global__ void band_bounds_kernel(const int32_t *__restrict__ kpos, const int32
 //    three long ones competing for the same SIMDs.
 //  * Every XCD takes at most cap = ceil(tiles / 8) tiles; the lightest tiles of an
 //    overfull XCD go to the XCDs that have room.
-// order[q * 8 + xcd] = tile | first offset << 24 (pre-filled with -1).  One workgroup; which of two
+// order[q * 8 + xcd] = tile | first offset << 24, -1 where no tile lands.  One workgroup; which of two
 // equally heavy tiles comes first depends on timing, the results do not.
 __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restrict__ perm,
                                                           const unsigned long long *__restrict__ block_masks,
@@ -196,6 +198,7 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t *__restr
     (&cursor[0][0])[i] = 0;
   }
   if (tid == 0) spill_count = 0;
+  for (int i = tid; i < cap * 8; i += 1024) order[i] = -1;     // (slots no tile lands in)
   __syncthreads();
   // entry of tile t in the table: t in the low 24 bits, the first offset the tile uses above
   // them (the kernel starts that offset's index load before it has seen the tile's masks)
@@ -290,11 +293,6 @@ __global__ void band_cells_kernel(const int32_t *__restrict__ band_start, int k_
     rank += before ? 1 : 0;
   }
   cells[(size_t)blockIdx.z * bands * k_vol + rank * 8 + x] = (c % k_vol) * 65536 + (c / k_vol) * 8 + x;
-}
-
-__global__ void iota_kernel(int32_t *__restrict__ p, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = i;
 }
 
 // out[k][pos] = in[k][perm[pos]]
@@ -476,7 +474,6 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
           set_error("fgms_plan_create: reorder allocation failed");
           return fail(FGMS_E_NOMEM);
         }
-        row_masks_kernel<<<(unsigned)((n + 255) / 256), 256, 0, sd>>>(tab, (int)n, k_vol, tmp_mask[d]);
         // stable LSD radix sort over the k_vol significant bits of the masks
         unsigned long long *keys_out = nullptr;
         int32_t *rows_in = nullptr;
@@ -491,7 +488,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
         ok = ok && pool_alloc(&sort_tmp, sort_bytes, sd) == FGMS_OK;
         if (ok) tmp_more.push_back(sort_tmp);
         if (ok) {
-          iota_kernel<<<(unsigned)((n + 255) / 256), 256, 0, sd>>>(rows_in, (int)n);
+          row_masks_kernel<<<(unsigned)((n + 255) / 256), 256, 0, sd>>>(tab, (int)n, k_vol, tmp_mask[d], rows_in);
           ok = rocprim::radix_sort_pairs(sort_tmp, sort_bytes, tmp_mask[d], keys_out, rows_in, perm,
                                          (size_t)n, 0u, (unsigned)k_vol, sd) == hipSuccess;
         }
@@ -518,10 +515,6 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
           return fail(FGMS_E_NOMEM);
         }
         (d ? p->tile_grid_in : p->tile_grid_out) = cap * 8;
-        if ((rc = fill_i32(order, (size_t)cap * 8, -1, sd))) {
-          free_tmp();
-          return fail(rc);
-        }
         tile_order_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), sd>>>(
             perm, mask, (int)n, n_tiles, cap, num_cus() >= 8 ? num_cus() / 8 : 1, order);
       }
