@@ -102,6 +102,42 @@ def test_config1_full_size_against_oracle(capi, oracle):
     plan.close()
 
 
+# Every BASELINE configuration at the size it is benchmarked at, element by element against
+# the C oracle (cpu-check.py:121-127 compares whole outputs the same way).  These are the
+# launches that take the full-size-only paths: tile tables with XCD homes, first offsets
+# from the tile table, 128-column wave tiles, split bf16 at 200 k voxels, the scattered
+# wide layer's dispatch.
+FULL = [
+    # cfg, variant, arch80, passes
+    (2, "fp16", False, "f"), (2, None, False, "f"), (2, None, True, "f"),
+    (3, None, False, "fdw"),
+    (4, None, False, "fdw"), (4, "up", False, "fdw"),
+    (5, "wide", False, "f"), (5, "wide-fp32", False, "f"),
+    (5, "skinny", False, "fdw"), (5, "skinny-fp32", False, "fdw"),
+]
+
+
+@pytest.mark.parametrize("cfg,variant,arch80,passes", FULL,
+                         ids=["cfg%d-%s%s" % (c, v or "default", "-tf32" if a else "") for c, v, a, _ in FULL])
+@pytest.mark.parametrize("with_plan", [True, False], ids=["plan", "no-plan"])
+def test_configs_full_size_against_oracle(capi, oracle, cfg, variant, arch80, passes, with_plan):
+    L = clouds.config_case(cfg, variant, scale=1.0)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(0)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"]) if with_plan else None
+    mode = G.mode_of(L["in_feats"].dtype, arch80)
+    a = (L["knnz"], L["imap"], L["omap"])
+    out = G.run_fwd(capi, D, fused=True, arch80=arch80, plan=plan)
+    G.assert_close(out, oracle.c_fwd(L["in_feats"], L["kernel"], *a, L["n_out"]), mode, "fwd")
+    if "d" in passes:
+        gi, gw = G.run_bwd(capi, D, plan=plan, arch80=arch80)
+        G.assert_close(gi, oracle.c_dgrad(L["out_grad"], L["kernel"], *a, L["n_in"]), mode, "dgrad")
+        # (a weight-gradient element sums tens of thousands of pairs: the float64 formulation)
+        G.assert_close(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *a, L["k_vol"]), mode, "wgrad")
+    if plan is not None:
+        plan.close()
+
+
 @pytest.mark.parametrize("side,c,dtype,tol", [(100, 64, torch.float16, 2e-3), (96, 32, torch.float32, 2e-5)],
                          ids=["1M-fp16", "885k-fp32"])
 def test_dense_grid_built_and_convolved_on_the_device(capi, side, c, dtype, tol):

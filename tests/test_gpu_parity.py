@@ -237,15 +237,13 @@ def test_baseline_configs_scaled(capi, oracle, cfg, variant):
     check_all(capi, oracle, L, policy=0, use_plan=False)
 
 
-@pytest.mark.parametrize("arch80", [False, True], ids=["", "tf32-mode"])
-@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+@pytest.mark.parametrize("dtype,arch80", [(np.float32, False), (np.float32, True), (np.float16, False)],
+                         ids=["fp32", "fp32-tf32-mode", "fp16"])
 @pytest.mark.parametrize("shape", [(32, 32), (64, 64), (128, 128), (64, 128), (256, 256), (96, 32)], ids=lambda s: "%dx%d" % s)
 def test_pair_view(capi, oracle, shape, dtype, arch80):
     """Policy 5: forward and input gradient run the output-stationary kernel over the plan's
     pair view (pair lists padded per offset to whole 64-row blocks, atomic sums); dense
     submanifold map, strided map and a map with empty offsets."""
-    if arch80 and dtype == np.float16:
-        pytest.skip("the flag only concerns fp32 tensors")
     capi.set_kernel_policy(5)
     try:
         L = layer(14, shape[0], shape[1], dtype)
