@@ -16,7 +16,7 @@ F32, F16 = 0, 1
 SYMBOLS = [
     "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_plan_stats", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
-    "fgms_wgrad", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
+    "fgms_wgrad", "fgms_wgrad_static", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
     "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map",
 ]
 
@@ -52,6 +52,7 @@ def lib():
                            i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_dgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
     L.fgms_wgrad.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64, i32, vp, vp]
+    L.fgms_wgrad_static.argtypes = L.fgms_wgrad.argtypes
     L.fgms_build_kernel_map.argtypes = [vp, i64, vp, i64, vp, i32, i32, i32, vp, vp, i64, vp, vp,
                                         ctypes.POINTER(ctypes.c_int64), vp]
     L.fgms_build_kernel_map.restype = i32
@@ -264,6 +265,16 @@ def wgrad(in_feats, out_grad, kernel_grad, kpos, in_map, out_map, plan=None):
     for t, n in ((in_feats, "in_feats"), (out_grad, "out_feats_grad"), (kernel_grad, "kernel_grad")):
         _need(t, n, in_feats.dtype)
     _check(lib().fgms_wgrad(
+        _p(in_feats), _p(out_grad), _p(kernel_grad), _p(kpos), _p(in_map), _p(out_map),
+        in_feats.shape[0], out_grad.shape[0], kernel_grad.shape[1], kernel_grad.shape[2],
+        kernel_grad.shape[0], in_map.numel(), _dtype(in_feats), _ph(plan), _stream()))
+
+
+def wgrad_static(in_feats, out_grad, kernel_grad, kpos, in_map, out_map, plan=None):
+    """fgms_wgrad_static: the weight gradient without any device allocation."""
+    for t, n in ((in_feats, "in_feats"), (out_grad, "out_feats_grad"), (kernel_grad, "kernel_grad")):
+        _need(t, n, in_feats.dtype)
+    _check(lib().fgms_wgrad_static(
         _p(in_feats), _p(out_grad), _p(kernel_grad), _p(kpos), _p(in_map), _p(out_map),
         in_feats.shape[0], out_grad.shape[0], kernel_grad.shape[1], kernel_grad.shape[2],
         kernel_grad.shape[0], in_map.numel(), _dtype(in_feats), _ph(plan), _stream()))

@@ -469,6 +469,22 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
   return run_wgrad(a);
 }
 
+int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *kernel_grad,
+                      const int32_t *kpos, const int32_t *in_map, const int32_t *out_map, int64_t n_in,
+                      int64_t n_out, int c_in, int c_out, int k_vol, int64_t n_pairs, int dtype,
+                      fgms_plan_t *plan, void *stream) {
+  int rc = check_common(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
+                        c_in, c_out, k_vol, n_pairs, dtype);
+  if (rc) return rc;
+  WgradArgs a{};
+  a.in = in_feats; a.gout = out_feats_grad; a.gw = kernel_grad; a.kpos = kpos;
+  a.imap = in_map; a.omap = out_map; a.n_in = n_in; a.n_out = n_out; a.c_in = c_in;
+  a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
+  a.stream = (hipStream_t)stream;
+  a.plan = (const Plan *)plan;
+  return wgrad_static(a);
+}
+
 int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kernel, int sum_nnz,
              void *in_feats_grad, void *kernel_grad, const int32_t *kpos, const int32_t *qkpos,
              const int32_t *in_map, const int32_t *out_map, int separate_mid, int arch80,

@@ -87,6 +87,9 @@ struct WgradArgs {
   // MFMA kernels, fp16: do not launch the fp32 -> fp16 flush of the accumulator; describe
   // it in *deferred_flush instead, for the caller to attach to its next launch
   SideJob *deferred_flush;
+  // MFMA kernels, fp16: use this fp32 accumulator (k_vol * c_in * c_out floats, all zero)
+  // instead of the stream's workspace; nothing is allocated then
+  float *acc_override;
 };
 
 // Plan: neighbour tables built from the pair lists.
@@ -174,6 +177,9 @@ int num_cus();         // compute units of the current device
 int launch_mfma_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);
+// The MFMA / skinny weight gradient with its fp32 accumulator in a static device array: no
+// allocation of any kind.
+int wgrad_static(WgradArgs a);
 // Describes the weight re-layout the output-stationary kernel needs for `a` as a side job
 // (nothing is launched) and returns where the packed weights will be.
 int planned_pack_job(const GmsArgs &a, SideJob *job, const void **packed);

@@ -20,6 +20,9 @@
 
 #include <stdlib.h>
 
+#include <map>
+#include <mutex>
+
 #include "fgms_device.h"
 #include "fgms_internal.h"
 #include "fgms_wgrad_bodies.h"
@@ -428,6 +431,10 @@ int wgrad_accumulator(const WgradArgs &a, float **acc32) {
     *acc32 = (float *)a.gw;
     return FGMS_OK;
   }
+  if (a.acc_override) {
+    *acc32 = a.acc_override;
+    return FGMS_OK;
+  }
   // partial sums of all workgroups meet in fp32 and are rounded to fp16 once.
   // The accumulator is zero-filled when it is (re)allocated and left zero by
   // every call, so no fill launch is needed per call.
@@ -455,7 +462,9 @@ int launch_mfma_wgrad(const WgradArgs &a) {
   if (rc != FGMS_OK) return rc;
   if (a.dtype != FGMS_F16) return dispatch<float>(a, acc32);
   if ((rc = dispatch<__half>(a, acc32))) {
-    (void)launch_fill_zero(acc32, workspace_bytes(a.stream, 1), a.stream);
+    const size_t bytes = a.acc_override ? (size_t)a.k_vol * a.c_in * a.c_out * sizeof(float)
+                                        : workspace_bytes(a.stream, 1);
+    (void)launch_fill_zero(acc32, bytes, a.stream);
     return rc;
   }
   if (a.deferred_flush) {
@@ -473,6 +482,65 @@ int launch_mfma_wgrad(const WgradArgs &a) {
     return FGMS_OK;
   }
   return wgrad_finish(a, acc32);
+}
+
+// ---------------------------------------------------------------------------
+// The weight gradient for callers that cannot allocate (code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc): the fp32 accumulator of the fp16 path
+// lives in a file-scope device array instead of the stream's grown-on-demand workspace.
+// Every GPU holds its own copy of the array at its own address until the process ends; the
+// array's name is only a host-side handle, so its device address is asked for once per
+// device and kept.
+constexpr size_t kScratchFloats = (size_t)2 << 20;       // 8 MiB: 27 offsets of 256 x 256 fit
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+namespace {
+std::mutex g_scratch_mutex;
+std::map<int, float *> g_scratch_ptr;       // device -> address of that device's copy
+
+int scratch_address(float **ptr) {
+  int dev = 0;
+  FGMS_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  auto it = g_scratch_ptr.find(dev);
+  if (it != g_scratch_ptr.end()) {
+    *ptr = it->second;
+    return FGMS_OK;
+  }
+  float *p = nullptr;
+  FGMS_HIP_TRY(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+  g_scratch_ptr[dev] = p;
+  *ptr = p;
+  return FGMS_OK;
+}
+}  // namespace
+
+int wgrad_static(WgradArgs a) {
+  if (a.n_pairs == 0) return FGMS_OK;
+  if (kernel_policy() == 1 || !mfma_wgrad_supported(a)) {
+    set_error("fgms_wgrad_static: only the shapes of the MFMA / skinny weight-gradient kernels "
+              "(channel counts that are multiples of 32, or 4/8/16 -> 16/32/64; 16-byte aligned rows)");
+    return FGMS_E_INVALID;
+  }
+  const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+  if (a.dtype == FGMS_F16) {
+    if (n > kScratchFloats) {
+      set_error("fgms_wgrad_static: k_vol * c_in * c_out = %zu exceeds the static accumulator's %zu floats",
+                n, kScratchFloats);
+      return FGMS_E_INVALID;
+    }
+    float *ptr = nullptr;
+    int rc = scratch_address(&ptr);
+    if (rc != FGMS_OK) return rc;
+    // the array keeps what the last call left (a failed or overlapping call may have left
+    // sums behind): the part this call uses starts from zero
+    if ((rc = launch_fill_zero(ptr, n * sizeof(float), a.stream))) return rc;
+    a.acc_override = ptr;
+  }
+  a.side = SideJob{};
+  a.deferred_flush = nullptr;
+  if (a.plan) a.plan->last_stream = a.stream;
+  return launch_mfma_wgrad(a);
 }
 
 }  // namespace fgms

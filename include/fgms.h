@@ -145,6 +145,24 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
                int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
                int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
 
+/*
+ * fgms_wgrad for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * Same arguments and results as fgms_wgrad, but the fp32 accumulator that the fp16 weight
+ * gradient sums in lives in a static device array inside the library (8 MiB per GPU, held
+ * until the process ends) instead of a workspace grown on demand, and the call makes no
+ * hipMalloc / hipFree or any other allocating call.  Limits: fp16 needs
+ * k_vol * c_in * c_out <= 2 097 152 (27 offsets of 256 x 256 fit); only the shapes of the
+ * MFMA and skinny kernels (channel counts that are multiples of 32, or 4/8/16 -> 16/32/64,
+ * 16-byte aligned rows) -- anything else returns FGMS_E_INVALID instead of falling back to a
+ * kernel that would need a workspace.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (two streams, two threads) race; calls on one stream do not.
+ */
+int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *kernel_grad,
+                      const int32_t *kpos, const int32_t *in_map, const int32_t *out_map,
+                      int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
+                      int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
+
 /* Selects kernels by hand for tests and profiling: 0 = automatic dispatch,
  * 1 = force the generic (non-MFMA) kernels, 2 = force the pair-stationary MFMA
  * kernels even when a usable plan is passed, 3 = automatic dispatch but the
