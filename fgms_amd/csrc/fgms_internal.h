@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "../../include/fgms.h"
 
 namespace fgms {
@@ -92,6 +94,19 @@ struct WgradArgs {
   float *acc_override;
 };
 
+// One direction of a plan's tile tables for the kernels that keep a tile's neighbourhood in
+// LDS (fgms_halo.hip): destination rows in a spatially compact order, cut into tiles of 256.
+struct HaloSide {
+  int32_t *order;               // [n_tiles * 256] position -> destination row, -1 = padding
+  int32_t *rows;                // [n_tiles][list_cap] the tile's distinct source rows, in source order
+  int32_t *count;               // [n_tiles] how many
+  unsigned short *lnbr;         // [k_vol][n_tiles * 256] index into the tile's list, 0xFFFF = no neighbour
+  unsigned long long *mask32;   // [n_tiles * 8] offsets in use per block of 32 positions
+  int n_tiles, list_cap;
+  int64_t extra_rounds;         // sum over tiles of the LDS rounds beyond the first
+  bool ok;                      // built and every tile's list fitted list_cap
+};
+
 // Plan: neighbour tables built from the pair lists.
 struct Plan {
   int device;
@@ -142,6 +157,7 @@ struct Plan {
   int32_t *pv_in, *pv_out;        // [pv_rows]
   unsigned long long *pv_mask;    // [pv_rows / 64]
   int64_t pv_rows;                // a multiple of 256
+  HaloSide halo[2];   // [0] forward (destination = output rows), [1] input gradient
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -195,6 +211,14 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p);
 // The same kernel over the plan's pair view (no wasted row slots, atomic adds).
 bool pair_view_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_pair_view_gms(const GmsArgs &a, const Plan *p);
+// Tile tables of the LDS-neighbourhood kernels (fgms_halo.hip).
+int halo_morton_order(const int32_t *coords, int64_t n, int coord_bits, int32_t **order, int32_t **inv,
+                      std::vector<void *> *tmp, hipStream_t s);
+int halo_build(Plan *p, int d, const int32_t *nbr_by_row, const int32_t *order_dst, const int32_t *inv_src,
+               const int32_t *order_src, int *flags, hipStream_t s);
+void halo_release(Plan *p);
+bool halo_gms_supported(const GmsArgs &a, const Plan *p);
+int launch_halo_gms(const GmsArgs &a, const Plan *p);
 int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
                      const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
                      int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,

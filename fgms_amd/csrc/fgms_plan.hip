@@ -336,11 +336,10 @@ int fill_i32(int32_t *p, size_t n, int32_t v, hipStream_t s) {
 
 using namespace fgms;
 
-extern "C" {
-
-int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
-                     const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
-                     int64_t n_pairs, void *stream) {
+namespace fgms {
+int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
+                const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
+                const int32_t *in_coords, const int32_t *out_coords, int coord_bits, void *stream) {
   if (!plan_out) {
     set_error("plan output pointer is null");
     return FGMS_E_INVALID;
@@ -361,6 +360,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->tile_out = p->tile_in = nullptr; p->tile_grid_out = p->tile_grid_in = 0;
   p->fwd_ok = p->dgrad_ok = false;
   p->pv_in = p->pv_out = nullptr; p->pv_mask = nullptr; p->pv_rows = 0;
+  p->halo[0] = p->halo[1] = HaloSide{};
   p->last_stream = s;
   int *flags = nullptr;
   int rc = FGMS_OK;
@@ -394,19 +394,37 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       pool_alloc((void **)&p->mask_in, (bi ? bi : 1) * sizeof(unsigned long long), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), s) != FGMS_OK ||
       pool_alloc((void **)&p->band_cells, (size_t)4 * k_vol * p->band_count * sizeof(int32_t), s) != FGMS_OK ||
-      pool_alloc((void **)&flags, 6 * sizeof(int), s) != FGMS_OK) {
+      pool_alloc((void **)&flags, 10 * sizeof(int), s) != FGMS_OK) {
     set_error("fgms_plan_create: table allocation failed");
     return fail(FGMS_E_NOMEM);
   }
   if ((rc = fill_i32(p->nbr_out, so, -1, s))) return fail(rc);
   if ((rc = fill_i32(p->nbr_in, si, -1, s))) return fail(rc);
-  if ((rc = fill_i32(flags, 6, 0, s))) return fail(rc);
+  if ((rc = fill_i32(flags, 10, 0, s))) return fail(rc);
   if (n_pairs > 0) {
     build_tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
         kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, p->nbr_out, p->nbr_in, flags);
     if (hipGetLastError() != hipSuccess) {
       set_error("fgms_plan_create: table build launch failed");
       return fail(FGMS_E_HIP);
+    }
+  }
+  // Row orders for the LDS-neighbourhood kernels: Morton order of the voxel coordinates where
+  // the caller supplies them (one order serves both sides of a submanifold map).
+  std::vector<void *> tmp_more;
+  int32_t *ord[2] = {nullptr, nullptr}, *inv[2] = {nullptr, nullptr};   // [0] output side, [1] input side
+  if (k_vol <= 64 && out_coords && in_coords) {
+    if ((rc = halo_morton_order(out_coords, n_out, coord_bits, &ord[0], &inv[0], &tmp_more, s)) == FGMS_OK) {
+      if (in_coords == out_coords && n_in == n_out) {
+        ord[1] = ord[0];
+        inv[1] = inv[0];
+      } else {
+        rc = halo_morton_order(in_coords, n_in, coord_bits, &ord[1], &inv[1], &tmp_more, s);
+      }
+    }
+    if (rc != FGMS_OK) {
+      for (void *q : tmp_more) pool_free(q, s, false);
+      return fail(rc);
     }
   }
   // fork: the input side's chain waits for the tables only
@@ -435,7 +453,6 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   // stream synchronisation below.
   int32_t *tmp_tab[2] = {nullptr, nullptr};
   unsigned long long *tmp_mask[2] = {nullptr, nullptr};
-  std::vector<void *> tmp_more;
   auto free_tmp = [&]() {
     if (s2 && !synced) {
       // work of the side stream may still use the temporaries: drain both streams first
@@ -518,6 +535,11 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
         tile_order_kernel<<<1, 1024, (size_t)n_tiles * sizeof(int32_t), sd>>>(
             perm, mask, (int)n, n_tiles, cap, num_cus() >= 8 ? num_cus() / 8 : 1, order);
       }
+      // tile tables of the LDS-neighbourhood kernels, from the table by destination row
+      if ((rc = halo_build(p, d, tmp_tab[d] ? tmp_tab[d] : tab, ord[d], inv[1 - d], ord[1 - d], flags + 6 + 2 * d, sd))) {
+        free_tmp();
+        return fail(rc);
+      }
     }
     if (s2 && (hipEventRecord(joined, s2) != hipSuccess || hipStreamWaitEvent(s, joined, 0) != hipSuccess)) {
       free_tmp();
@@ -530,7 +552,7 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
       return fail(FGMS_E_HIP);
     }
   }
-  int h[6] = {0, 0, 0, 0, 0, 0};
+  int h[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   if (hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
       hipStreamSynchronize(s) != hipSuccess) {
     free_tmp();
@@ -550,6 +572,10 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   p->bands_ok = !h[3];
   p->stages_out = h[4];
   p->stages_in = h[5];
+  for (int d = 0; d < 2; ++d) {
+    p->halo[d].ok = p->halo[d].order != nullptr && !h[6 + 2 * d];
+    p->halo[d].extra_rounds = h[7 + 2 * d];
+  }
   // The pair view, for maps sparse enough that some layer would take it (fp32 layers prefer
   // it from about 1 + 45 / channels row slots per pair on, never below 1.4): built after the
   // counts are known, with a synchronisation of its own, so that dense maps pay nothing.
@@ -578,10 +604,32 @@ int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t 
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
 }
+}  // namespace fgms
+
+extern "C" {
+
+int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
+                     const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
+                     int64_t n_pairs, void *stream) {
+  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, nullptr, nullptr, 0, stream);
+}
+
+int fgms_plan_create_coords(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
+                            const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
+                            int64_t n_pairs, const int32_t *in_coords, const int32_t *out_coords,
+                            int coord_bits, void *stream) {
+  if ((n_in > 0 && !in_coords) || (n_out > 0 && !out_coords) || coord_bits < 0 || coord_bits > 21) {
+    set_error("fgms_plan_create_coords: null coordinates or coord_bits outside 0..21");
+    return FGMS_E_INVALID;
+  }
+  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, in_coords, out_coords,
+                     coord_bits, stream);
+}
 
 void fgms_plan_destroy(fgms_plan_t *plan) {
   Plan *p = (Plan *)plan;
   if (!p) return;
+  halo_release(p);
   if (p->nbr_out) pool_free(p->nbr_out, p->last_stream, false);
   if (p->nbr_in) pool_free(p->nbr_in, p->last_stream, false);
   if (p->mask_out) pool_free(p->mask_out, p->last_stream, false);
