@@ -13,6 +13,19 @@ Prints ONE JSON line:  effective TFLOP/s = passes * 2 * M * Cin * Cout / t with
 M the real (unpadded) pair count, a roofline object for the dominant kernel
 (duration from HIP events on the launch stream) and the CPU baseline (the C
 restatement of cpu-check.py / cpu-check-back.py on this box's host cores).
+
+Order of a run: per-kernel event pass, plan / map-build timings and the second
+surface first (they double as clock warm-up: a run that asks for few steps is
+otherwise measured during the first milliseconds after idle), then the W warm-up
+steps, then the timed region of exactly K steps, then the CPU baseline.
+
+`value` is the step through the C ABI with an explicit plan built before the timed
+region; what building the plan costs is in the same line (`plan`): its wall-clock
+cost per call, the step time when it is paid once per 1 / 4 / 16 layer-steps (a
+point cloud changes every iteration, a kernel map serves the handful of layers of
+one resolution), and the step time without any plan.  `surface_backend` is the
+same step through the python extension FGMS.backend (the reference's three
+functions; plan found in its cache).
 """
 import argparse
 import json
@@ -75,12 +88,15 @@ def compulsory_bytes(L):
 
 def cpu_baseline(name, budget_s=12.0):
     """Times the CPU oracle (OpenMP, this box's host cores) on a bounded sample of
-    the same workload and returns effective TFLOP/s."""
+    the same workload and returns effective TFLOP/s, with all the threads the box
+    grants and with one."""
     from oracle import fgms_oracle as oracle
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    host_cores = os.cpu_count() or 1
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, host_cores)
     threads = max(1, min(threads, oracle.max_threads() if oracle.max_threads() > 0 else threads))
+    all_threads = threads
 
-    def run(scale, repeats=1):
+    def run(scale, repeats=1, threads=all_threads):
         L, passes, _ = make_case(name, scale)
         args = (L["knnz"], L["imap"], L["omap"])
         t0 = time.perf_counter()
@@ -104,12 +120,32 @@ def cpu_baseline(name, budget_s=12.0):
         repeats = max(1, min(200, int(budget_s / max(dt / scale * want, 1e-3))))
         scale = want
         dt, flops, L = run(scale, repeats)
+    # one thread, on a sample a sixteenth of that (about the same time again at most)
+    dt1, flops1, L1 = run(max(scale / 16.0, 0.01), 1, threads=1)
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "host_cores": host_cores, "threads": threads,
+        "value_1_thread": flops1 / dt1 / 1e12,
+        "sample_1_thread": "%d voxels, %d pairs, one pass each, %.1f s" % (L1["n_in"], len(L1["imap"]), dt1),
         "sample": "%s at %.0f%% of the voxels (%d voxels, %d pairs), %d x one pass each of %s, %.1f s"
                   % (name.split("-")[0] + " cloud", scale * 100, L["n_in"], len(L["imap"]), repeats,
                      "+".join(WORKLOADS[name][2]), dt),
     }
+
+
+TRAFFIC_SOURCE = ("profiles/hbm_traffic.json: rocprofv3 FETCH_SIZE / WRITE_SIZE of an earlier profiled run of this "
+                  "command (KiB per dispatch, scaled by a plain copy of known size); not measured by this run")
+
+
+def to_dev(L):
+    """The numpy layer on the GPU (kernel_nnz stays on the host, as the reference reads it there)."""
+    import numpy as np
+    import torch
+    d = {}
+    for k, v in L.items():
+        d[k] = torch.from_numpy(v).cuda() if isinstance(v, np.ndarray) and k != "knnz" else v
+    d["knnz_host"] = torch.from_numpy(L["knnz"].astype(np.int32))
+    return d
 
 
 def measured_traffic(workload, kernel):
@@ -137,7 +173,13 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--scale", type=float, default=1.0, help="voxel-count scale (1.0 = the named size)")
     ap.add_argument("--map-build", action="store_true",
-                    help="also time the device kernel-map builder and the plan build on the headline cloud")
+                    help="also report the device kernel-map builder's kernels (the map and plan build costs are always reported)")
+    ap.add_argument("--surface", default="cabi", choices=["cabi", "backend"],
+                    help="what `value` times: the C ABI with an explicit plan (default) or the python "
+                         "extension FGMS.backend (plan from its cache); the other one is reported next to it")
+    ap.add_argument("--coords-plan", action="store_true",
+                    help="build the plan with the voxel coordinates (fgms_plan_create_coords) and run the "
+                         "LDS-neighbourhood kernel where it applies (kernel policy 6)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run plain 256 MiB device copies (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -148,14 +190,32 @@ def main():
 
     import torch
     from fgms_amd import capi
-    from tests.gpu_util import to_dev
+    import FGMS.backend as backend
 
     capi.lib()  # fails loudly if the HIP library is missing
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     L, passes, arch80 = make_case(args.workload, args.scale)
     D = to_dev(L)
+    if args.coords_plan:
+        args.policy = 6
     capi.set_kernel_policy(args.policy)
-    plan = None if args.no_plan else capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    backend.fgms_set_kernel_policy(args.policy)
+    backend.fgms_plan_cache(not args.no_plan)
+    coords = None
+    if args.coords_plan:
+        import numpy as np
+        from fgms_amd import clouds
+        if WORKLOADS[args.workload][0] != 2 and not args.workload.startswith("cfg5-skinny"):
+            print("bench.py: --coords-plan is wired for the submanifold layers over the indoor cloud", file=sys.stderr)
+            sys.exit(2)
+        coords = torch.from_numpy(np.ascontiguousarray(
+            clouds.cloud_indoor(clouds.rng_for(2), target=int(200000 * args.scale)), dtype=np.int32)).cuda()
+
+    def make_plan():
+        return capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"],
+                         in_coords=coords, out_coords=coords, coord_bits=9 if coords is not None else 0)
+
+    plan = None if args.no_plan else make_plan()
     dt = D["in_feats"].dtype
     out = torch.zeros(D["n_out"], D["c_out"], dtype=dt, device="cuda")
     gi = torch.zeros(D["n_in"], D["c_in"], dtype=dt, device="cuda")
@@ -163,7 +223,7 @@ def main():
     m = len(L["imap"])
     flops_pass = 2.0 * m * L["c_in"] * L["c_out"]
 
-    def step():
+    def step_cabi(plan=plan):
         if "fwd" in passes:
             capi.fusion_fwd(D["in_feats"], D["kernel"], 0, out, D["kpos"], None, D["imap"], D["omap"],
                             False, arch80, plan=plan)
@@ -177,6 +237,31 @@ def main():
             if "wgrad" in passes:
                 capi.wgrad(D["in_feats"], D["out_grad"], gw, D["kpos"], D["imap"], D["omap"], plan=plan)
 
+    qkpos = torch.zeros_like(D["kpos"])      # (accepted and ignored: tiles are derived from kpos)
+    backend_ok = ("dgrad" in passes) == ("wgrad" in passes)     # the extension has the reference's three functions only
+
+    def step_backend():
+        if "fwd" in passes:
+            backend.fgms_fusion_fwd_cuda(D["in_feats"], D["kernel"], 0, out, D["kpos"], qkpos, D["imap"], D["omap"],
+                                         False, arch80)
+        if "dgrad" in passes:
+            backend.fgms_bwd_cuda(D["out_grad"], D["in_feats"], D["kernel"], 0, gi, gw, D["kpos"], qkpos,
+                                  D["imap"], D["omap"], False, arch80)
+
+    if args.surface == "backend" and not backend_ok:
+        print("bench.py: FGMS.backend has no entry point for one gradient alone", file=sys.stderr)
+        sys.exit(2)
+    step = step_backend if args.surface == "backend" else step_cabi
+    other = step_cabi if args.surface == "backend" else (step_backend if backend_ok and coords is None else None)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        a = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - a) * 1e3 / n
+
     if args.copy_calib:
         a_ = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
         b_ = torch.empty_like(a_)
@@ -184,23 +269,15 @@ def main():
             b_.copy_(a_)
         torch.cuda.synchronize()
         del a_, b_
-    for _ in range(args.warmup):
+    # per-kernel durations: steps with a HIP event pair around every kernel launch (recorded on
+    # the launch stream by the library).  Kept out of the timed region below because the ten
+    # event records per step cost 20-30 us of stream time themselves; run first, so that they
+    # also bring the clocks up for runs that ask for few steps.
+    for _ in range(5):
         step()
-    out.zero_(); gi.zero_(); gw.zero_()
-    torch.cuda.synchronize()
-    # the timed region: exactly K steps, nothing else on the stream
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-
-    # the same K steps again with a HIP event pair around every kernel launch (recorded on
-    # the launch stream by the library): per-kernel durations.  Kept out of the timed region
-    # above because the ten event records per step cost 20-30 us of stream time themselves.
     capi.profile_reset()
     capi.profile_enable(True)
-    prof_steps = min(args.steps, 200)
+    prof_steps = max(min(args.steps, 200), 50)
     tp0 = time.perf_counter()
     for _ in range(prof_steps):
         step()
@@ -231,16 +308,30 @@ def main():
         gather_floor["what"] = ("fgms_probe_gather: the same neighbour-table gathers as the planned kernel, "
                                 "nothing else (no weights, MFMA, LDS or result rows), all wave slots in use")
 
-    # the steps before the path: pair lists from coordinates, plan from pair lists
+    # the steps before the path: pair lists from coordinates (the indoor cloud's workloads), plan
+    # from pair lists; the same step with no plan at all; the other surface
+    import numpy as np
+    from fgms_amd import clouds
+    plan_cost = {}
+    t_plan = None
+    if not args.no_plan:
+        for _ in range(3):
+            make_plan().close()
+        torch.cuda.synchronize()
+        tb = time.perf_counter()
+        for _ in range(10):
+            make_plan().close()
+        torch.cuda.synchronize()
+        t_plan = (time.perf_counter() - tb) / 10 * 1e3
+        plan_cost["plan_create_ms"] = t_plan
     map_build = None
-    if args.map_build:
-        import numpy as np
-        from fgms_amd import clouds
+    cfg_id = WORKLOADS[args.workload][0]
+    if cfg_id in (2, 5) and "wide" not in args.workload and args.scale == 1.0:
         vox = torch.from_numpy(np.ascontiguousarray(clouds.indoor_cloud())).cuda()
         offs = clouds.offsets_cube(3)
         for _ in range(3):
             capi.build_kernel_map(vox, vox, offs)
-        capi.profile_enable(True)
+        capi.profile_enable(args.map_build)
         torch.cuda.synchronize()
         tb = time.perf_counter()
         for _ in range(10):
@@ -248,26 +339,58 @@ def main():
         torch.cuda.synchronize()
         t_map = (time.perf_counter() - tb) / 10
         capi.profile_enable(False)
-        pr = {}
-        for name, ms in capi.profile_records():
-            pr.setdefault(name, []).append(ms)
-        capi.profile_reset()
-        tb = time.perf_counter()
-        for _ in range(10):
-            capi.Plan(kp_, im_, om_, vox.shape[0], vox.shape[0]).close()
-        torch.cuda.synchronize()
-        t_plan = (time.perf_counter() - tb) / 10
-        nbytes = 2 * vox.numel() * 4 + 2 * im_.numel() * 4     # coordinates read, pair lists written
-        k_ms = {k: sum(v) / len(v) for k, v in pr.items()}
-        map_build = {"voxels": int(vox.shape[0]), "pairs": int(im_.numel()), "k_vol": 27,
-                     "build_kernel_map_ms": t_map * 1e3, "kernels_ms": k_ms,
-                     "algorithmic_GBs": nbytes / (sum(k_ms.values()) * 1e-3) / 1e9,
-                     "plan_create_ms": t_plan * 1e3,
-                     "note": "wall clock per call incl. temporary allocations and the one synchronisation; "
-                             "algorithmic bytes = coordinates read + pair lists written"}
+        plan_cost["build_kernel_map_ms"] = t_map * 1e3
+        if args.map_build:
+            pr = {}
+            for name, ms in capi.profile_records():
+                pr.setdefault(name, []).append(ms)
+            capi.profile_reset()
+            nbytes = 2 * vox.numel() * 4 + 2 * im_.numel() * 4     # coordinates read, pair lists written
+            k_ms = {k: sum(v) / len(v) for k, v in pr.items()}
+            map_build = {"voxels": int(vox.shape[0]), "pairs": int(im_.numel()), "k_vol": 27,
+                         "build_kernel_map_ms": t_map * 1e3, "kernels_ms": k_ms,
+                         "algorithmic_GBs": nbytes / (sum(k_ms.values()) * 1e-3) / 1e9,
+                         "plan_create_ms": t_plan,
+                         "note": "wall clock per call incl. temporary allocations and the one synchronisation; "
+                                 "algorithmic bytes = coordinates read + pair lists written"}
+        del vox, im_, om_
+    if not args.no_plan and args.surface == "cabi":
+        capi.set_kernel_policy(0 if args.policy == 6 else args.policy)
+        n_np = max(5, min(50, args.steps))
+        step_cabi(plan=None)
+        plan_cost["no_plan_ms_per_step"] = timed(lambda: step_cabi(plan=None), n_np)
+        capi.set_kernel_policy(args.policy)
+    surface_other = None
+    if other is not None:
+        n_o = max(20, min(200, args.steps))
+        for _ in range(5):
+            other()
+        surface_other = {"ms_per_step": timed(other, n_o), "steps": n_o}
+
+    # W warm-up steps, then the timed region: exactly K steps, nothing else on the stream
+    for _ in range(args.warmup):
+        step()
+    out.zero_(); gi.zero_(); gw.zero_()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    value = len(passes) * flops_pass / (ms_per_step * 1e-3) / 1e12
+    step_flops = len(passes) * flops_pass
+    value = step_flops / (ms_per_step * 1e-3) / 1e12
+    if t_plan is not None:
+        # one plan build per `reuse` layer-steps (a layer-step = this workload's step)
+        plan_cost["incl_plan"] = {
+            "reuse_%d" % r: {"ms_per_step": ms_per_step + t_plan / r,
+                             "value": step_flops / ((ms_per_step + t_plan / r) * 1e-3) / 1e12}
+            for r in (1, 4, 16)}
+    if "no_plan_ms_per_step" in plan_cost:
+        plan_cost["no_plan_value"] = step_flops / (plan_cost["no_plan_ms_per_step"] * 1e-3) / 1e12
+    if surface_other is not None:
+        surface_other["value"] = step_flops / (surface_other["ms_per_step"] * 1e-3) / 1e12
 
     # per-kernel averages from the HIP events recorded on the launch stream
     per = {}
@@ -282,16 +405,20 @@ def main():
         skinny = min(L["c_in"], L["c_out"]) <= 16
         if skinny:
             which = "dgrad" if "dgrad" in dom else "fwd"
-            ach = dataflow_bytes(L, which) / avg_s / 1e9
+            # HBM-bound launch: the algorithmic bytes are the ones no kernel can avoid (every
+            # tensor once); a kernel that keeps result rows on chip moves fewer bytes than the
+            # pair-list count (a row per pair), so that count is reported as a pricing only
+            traffic = measured_traffic(args.workload, dom)
+            ach = compulsory_bytes(L) / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": PEAK_HBM_GBS,
-                        "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": measured_traffic(args.workload, dom),
+                        "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": traffic,
+                        "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+                        "traffic_GBs": traffic / avg_s / 1e9 if traffic is not None else None,
                         "avg_kernel_ms": kernels[dom]["avg_ms"],
-                        # `achieved` prices the launch as pair-list dataflow (a row per pair); a
-                        # kernel that keeps rows on chip moves less and can exceed the peak by
-                        # that count.  The same launch against the bytes no kernel can avoid:
-                        "compulsory_bytes": compulsory_bytes(L),
-                        "compulsory_GBs": compulsory_bytes(L) / avg_s / 1e9,
-                        "compulsory_frac": compulsory_bytes(L) / avg_s / 1e9 / PEAK_HBM_GBS}
+                        "algorithmic_bytes": compulsory_bytes(L),
+                        "algorithmic_bytes_what": "(N_in*Cin + N_out*Cout)*s + 8*M + K*Cin*Cout*s: every tensor once",
+                        "pair_list_pricing_bytes": dataflow_bytes(L, which),
+                        "pair_list_pricing_GBs": dataflow_bytes(L, which) / avg_s / 1e9}
         else:
             # the backward call's single launch computes both gradients
             parts = ("dgrad", "wgrad") if dom.startswith("bwd_fused") else \
@@ -301,14 +428,18 @@ def main():
             factor, peak = (3, PEAK_TFLOPS["f16"]) if "bf16x3" in dom else (1, PEAK_TFLOPS[arith])
             ach = factor * len(parts) * flops_pass / avg_s / 1e12
             flow = sum(dataflow_bytes(L, w_) for w_ in parts)
+            traffic = measured_traffic(args.workload, dom)
             roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": peak,
-                        "unit": "TFLOP/s", "frac": ach / peak, "traffic": measured_traffic(args.workload, dom),
+                        "unit": "TFLOP/s", "frac": ach / peak, "traffic": traffic,
+                        "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
                         "mfma_flop_per_algorithmic_flop": factor,
                         "avg_kernel_ms": kernels[dom]["avg_ms"],
-                        # the same launch priced as pair-list dataflow bytes against HBM
                         "passes_in_kernel": list(parts),
-                        "dataflow_bytes": flow,
-                        "dataflow_GBs": flow / avg_s / 1e9}
+                        "algorithmic_flop": factor * len(parts) * flops_pass,
+                        # the same launch PRICED as pair-list bytes (a gathered row and a result row
+                        # per pair) -- a pricing, not traffic: caches serve the re-reads
+                        "pair_list_pricing_bytes": flow,
+                        "pair_list_pricing_GBs": flow / avg_s / 1e9}
 
     line = {
         "metric": "effective TFLOP/s (2*sum|map_k|*Cin*Cout/t), %s, %s"
@@ -319,12 +450,15 @@ def main():
         "vs_baseline": None, "dtype": arith, "data": "synthetic",
         "config": {"workload": args.workload, "voxels_in": L["n_in"], "voxels_out": L["n_out"],
                    "pairs": m, "k_vol": L["k_vol"], "c_in": L["c_in"], "c_out": L["c_out"],
-                   "plan": plan is not None, "policy": args.policy,
+                   "plan": plan is not None, "policy": args.policy, "surface": args.surface,
+                   "plan_with_coordinates": coords is not None,
                    "row_slots_per_pair": (round(plan.stats()["blocks_fwd"] * 64.0 / max(plan.stats()["pairs"], 1), 3)
                                           if plan is not None else None)},
         "kernels": kernels,
         "roofline": roofline,
         "gather_floor": gather_floor,
+        "plan": plan_cost or None,
+        ("surface_backend" if args.surface == "cabi" else "surface_cabi"): surface_other,
         "map_build": map_build,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload),
     }
