@@ -24,6 +24,12 @@
 // the bytes through L1: with 128 accumulator registers a CU holds 8 waves, and a tile's 14 us
 // are mostly memory round trips those few waves cannot cover (neighbourhood load 2.9 us, the
 // offsets' weight fetches 8 us for 1.9 us of MFMA work, reduction and row update 3.5 us).
+// A weight-stationary variant (one persistent workgroup per CU, every wave keeping the B
+// fragments of its three or four offsets in registers for the whole launch, per-tile sums
+// combined in LDS) was measured too: ds_add_f32 runs at about a lane per clock, 620 us per pass;
+// with plain stores in its place (wrong sums, timing only) still 75 us, because the compiler
+// waits for every outstanding direct-to-LDS load before any LDS access that follows it, which
+// undoes the double buffering of the neighbourhood rows.
 // So this path is opt-in: the tables are built by fgms_plan_create_coords only, and the
 // kernel runs under kernel policy 6 only.
 #include <stdlib.h>
@@ -41,7 +47,7 @@ namespace fgms {
 namespace {
 
 constexpr int kHaloTile = 128;    // destination rows per tile (4 blocks of 32)
-constexpr int kHaloCap = 320;     // neighbourhood rows resident in LDS per round
+constexpr int kHaloCap = 352;     // neighbourhood rows resident in LDS per round
 constexpr int kHaloThreads = 256; // the kernel's workgroup
 constexpr int kBuildThreads = kHaloTile;   // the plan kernel's: one thread per position of a tile
 constexpr int kHashSlots = 8192;  // >= 64 offsets x 128 rows; 27 x 256 = 6 912 keys fit too
