@@ -49,8 +49,15 @@ class KernelMap:
         return cls(in_map, out_map, knnz, in_coords.shape[0], out_coords.shape[0])
 
     def transposed(self):
-        """The map of the transposed convolution: the same pairs, roles swapped."""
-        return KernelMap(self.out_map, self.in_map, self.kernel_nnz, self.n_out, self.n_in)
+        """The map of the transposed convolution: the same pairs, roles swapped.  It keeps
+        this map's tensors (not copies), so ``FGMS.backend`` recognises the pair lists and lets
+        both maps share one plan."""
+        t = KernelMap.__new__(KernelMap)
+        t.k_vol, t.kernel_nnz = self.k_vol, self.kernel_nnz
+        t.in_map, t.out_map = self.out_map, self.in_map
+        t.kpos, t.qkpos, t.qsum = self.kpos, self.qkpos, self.qsum
+        t.n_in, t.n_out = self.n_out, self.n_in
+        return t
 
 
 class _SparseConvFunction(torch.autograd.Function):

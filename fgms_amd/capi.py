@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfgms_hip.so")
 
 F32, F16 = 0, 1
 SYMBOLS = [
-    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_create_coords", "fgms_plan_destroy",
+    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_create_coords", "fgms_plan_transposed", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_plan_stats", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_wgrad_static", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
     "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map",
@@ -40,6 +40,7 @@ def lib():
     L.fgms_last_error.restype = ctypes.c_char_p
     L.fgms_plan_create.argtypes = [ctypes.POINTER(vp), vp, vp, vp, i64, i64, i32, i64, vp]
     L.fgms_plan_create_coords.argtypes = [ctypes.POINTER(vp), vp, vp, vp, i64, i64, i32, i64, vp, vp, i32, vp]
+    L.fgms_plan_transposed.argtypes = [ctypes.POINTER(vp), vp]
     L.fgms_plan_destroy.argtypes = [vp]
     L.fgms_plan_destroy.restype = None
     L.fgms_plan_usable.argtypes = [vp, i32]
@@ -158,6 +159,15 @@ class Plan:
     @property
     def handle(self):
         return self._h
+
+    def transposed(self):
+        """A plan for the same pairs with in_map and out_map exchanged (the transposed
+        convolution's map); shares this plan's tables."""
+        view = Plan.__new__(Plan)
+        view._keep = (self,) + tuple(self._keep)
+        view._h = ctypes.c_void_p()
+        _check(lib().fgms_plan_transposed(ctypes.byref(view._h), self._h))
+        return view
 
     def usable(self, for_dgrad=False):
         return bool(lib().fgms_plan_usable(self._h, int(for_dgrad)))

@@ -59,6 +59,13 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   WsBuf &b = g_ws[WsKey{dev, stream, slot}];
   if (b.bytes < bytes) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
+      // growing would free a buffer that recorded kernels point at, and allocate under capture
+      set_error("a workspace of %zu bytes is needed while the stream is being captured: run the call once "
+                "outside the capture first", bytes);
+      return FGMS_E_INVALID;
+    }
     if (b.ptr) {
       // the old buffer may still be in use by work queued on this stream
       FGMS_HIP_TRY(hipStreamSynchronize(stream));
@@ -294,7 +301,7 @@ Route route_of(const GmsArgs &a, const Plan *plan) {
 }
 
 int run_gms(GmsArgs a, const Plan *plan) {
-  if (plan) plan->last_stream = a.stream;
+  if (plan) plan_touch(plan, a.stream);
   const bool dense = a.dense_k >= 0;
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
   switch (route_of(a, plan)) {
@@ -309,7 +316,7 @@ int run_gms(GmsArgs a, const Plan *plan) {
 
 int run_wgrad(const WgradArgs &a) {
   if (a.n_pairs == 0) return FGMS_OK;
-  if (a.plan) a.plan->last_stream = a.stream;
+  if (a.plan) plan_touch(a.plan, a.stream);
   if (g_policy != 1 && mfma_wgrad_supported(a)) return launch_mfma_wgrad(a);
   return launch_generic_wgrad(a);
 }
@@ -394,7 +401,9 @@ int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz, void 
     d.n_dense = n_out;
     if ((rc = run_gms(d, nullptr))) return rc;
   }
-  return run_gms(a, (const Plan *)plan);
+  const Plan *p = plan_resolve(plan, s, &rc);
+  if (rc) return rc;
+  return run_gms(a, p);
 }
 
 int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_feats,
@@ -430,7 +439,9 @@ int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_fe
   GmsArgs a = fwd_args(in_feats, kernel, out_feats, kernel_pos, in_map, out_map, n_in, n_out,
                        c_in, c_out, k_vol, total, dtype, s);
   a.reduced = arch80 != 0 && dtype == FGMS_F32;
-  if ((rc = run_gms(a, (const Plan *)plan))) return rc;
+  const Plan *p = plan_resolve(plan, s, &rc);
+  if (rc) return rc;
+  if ((rc = run_gms(a, p))) return rc;
   if (separate_mid) {
     GmsArgs d = a;
     d.gmap = d.smap = nullptr;
@@ -454,7 +465,9 @@ int fgms_dgrad(const void *out_feats_grad, const void *kernel, void *in_feats_gr
   a.n_src = n_out; a.n_dst = n_in; a.c_in = c_in; a.c_out = c_out; a.k_vol = k_vol;
   a.n_pairs = n_pairs; a.transpose_w = true; a.dense_k = -1; a.n_dense = 0; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
-  return run_gms(a, (const Plan *)plan);
+  const Plan *p = plan_resolve(plan, a.stream, &rc);
+  if (rc) return rc;
+  return run_gms(a, p);
 }
 
 int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_grad,
@@ -469,7 +482,8 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
   a.imap = in_map; a.omap = out_map; a.n_in = n_in; a.n_out = n_out; a.c_in = c_in;
   a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
-  a.plan = (const Plan *)plan;
+  a.plan = plan_resolve(plan, a.stream, &rc);
+  if (rc) return rc;
   return run_wgrad(a);
 }
 
@@ -485,7 +499,8 @@ int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *ke
   a.imap = in_map; a.omap = out_map; a.n_in = n_in; a.n_out = n_out; a.c_in = c_in;
   a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
-  a.plan = (const Plan *)plan;
+  a.plan = plan_resolve(plan, a.stream, &rc);
+  if (rc) return rc;
   return wgrad_static(a);
 }
 
@@ -501,7 +516,8 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
   if ((rc = check_common(in_feats, out_feats_grad, kernel_grad, kpos, in_map, out_map, n_in, n_out,
                          c_in, c_out, k_vol, n_pairs, dtype)))
     return rc;
-  const Plan *p = (const Plan *)plan;
+  const Plan *p = plan_resolve(plan, (hipStream_t)stream, &rc);
+  if (rc) return rc;
   GmsArgs d{};
   d.src = out_feats_grad; d.w = kernel; d.dst = in_feats_grad; d.kpos = kpos;
   d.gmap = out_map; d.smap = in_map;   // roles swap, as at backend/spconv.cu:460,559
@@ -521,7 +537,7 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
   // whose launch in turn also rounds the weight gradient's fp32 sums into the caller's
   // fp16 tensor.  (The two gradients do not depend on each other.)
   if (n_pairs > 0 && route_of(d, p) == Route::kRows && g_policy != 1 && mfma_wgrad_supported(w)) {
-    p->last_stream = d.stream;
+    plan_touch(p, d.stream);
     // one launch for both where the shapes allow (and a small one that rounds an fp16
     // weight gradient), else two
     bool fused = false;
@@ -562,12 +578,13 @@ int fgms_build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t 
 
 int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad, fgms_plan_t *plan,
                       void *stream) {
-  const Plan *p = (const Plan *)plan;
+  int prc = FGMS_OK;
+  const Plan *p = plan_resolve(plan, (hipStream_t)stream, &prc);
   if (!p || !feats || c_src <= 0 || (dtype != FGMS_F16 && dtype != FGMS_F32)) {
-    set_error("fgms_probe_gather: bad argument");
+    if (!prc) set_error("fgms_probe_gather: bad argument");
     return FGMS_E_INVALID;
   }
-  p->last_stream = (hipStream_t)stream;
+  plan_touch(p, (hipStream_t)stream);
   void *sink = nullptr;
   int rc = workspace_get((hipStream_t)stream, 3, 256, &sink);
   if (rc) return rc;

@@ -86,7 +86,8 @@ __global__ void invert_order_kernel(const int32_t *__restrict__ order, int n, in
 // One workgroup per tile of kHaloTile positions: (optionally) sorts the tile's rows by offset
 // mask, lists the distinct source rows of the tile in source-position order and renumbers
 // the neighbour table in positions of that list.
-//   nbr       [k_vol][n_dst]  by destination ROW: source row or -1
+//   nbr       [k_vol][n_dst]  by the plan's POSITION of the destination row: source row or -1
+//   plan_pos  [n_dst]         destination row -> that position (nullptr: identity)
 //   order_dst [n_dst]         position -> destination row (nullptr: identity)
 //   inv_src   [n_src]         source row -> source position (nullptr: identity)
 //   order_src [n_src]         source position -> source row (nullptr: identity)
@@ -94,7 +95,7 @@ __global__ void invert_order_kernel(const int32_t *__restrict__ order, int n, in
 //      lnbr [k_vol][n_tiles * kHaloTile], mask32 [n_tiles * kHaloTile / 32];
 //      flags[0] = 1 if some list did not fit, flags[1] += rounds beyond the first.
 __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
-    const int32_t *__restrict__ nbr, const int32_t *__restrict__ order_dst,
+    const int32_t *__restrict__ nbr, const int32_t *__restrict__ plan_pos, const int32_t *__restrict__ order_dst,
     const int32_t *__restrict__ inv_src, const int32_t *__restrict__ order_src, int n_dst, int k_vol,
     int sort_by_mask, int list_cap, int32_t *__restrict__ order_pad, int32_t *__restrict__ rows,
     int32_t *__restrict__ count, unsigned short *__restrict__ lnbr,
@@ -108,6 +109,7 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
   const int n_pad = gridDim.x * kHaloTile;
   const int p = tile * kHaloTile + tid;
   int row = p < n_dst ? (order_dst ? order_dst[p] : p) : -1;
+  int col = row >= 0 ? (plan_pos ? plan_pos[row] : row) : 0;      // the row's column of the table
   for (int i = tid; i < kHashSlots; i += kBuildThreads) table[i] = -1;
   for (int i = tid; i < 1024; i += kBuildThreads) list[i] = INT32_MAX;
   if (tid == 0) n_list = 0;
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
     // offsets none of its rows uses.  Ties keep their order (the key carries the position).
     unsigned long long m = 0;
     for (int k = 0; k < k_vol; ++k)
-      if (row >= 0 && nbr[(size_t)k * n_dst + row] >= 0) m |= 1ull << k;
+      if (row >= 0 && nbr[(size_t)k * n_dst + col] >= 0) m |= 1ull << k;
     skey[tid] = row >= 0 ? m : ~0ull;
     sval[tid] = row;
     __syncthreads();
@@ -142,12 +144,13 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
         __syncthreads();
       }
     row = sval[tid];
+    col = row >= 0 ? (plan_pos ? plan_pos[row] : row) : 0;
   }
   order_pad[p] = row;
   __syncthreads();
   // distinct source positions of the tile
   for (int k = 0; k < k_vol; ++k) {
-    const int g = row >= 0 ? nbr[(size_t)k * n_dst + row] : -1;
+    const int g = row >= 0 ? nbr[(size_t)k * n_dst + col] : -1;
     if (g < 0) continue;
     const int key = inv_src ? inv_src[g] : g;
     unsigned slot = ((unsigned)key * 2654435761u) >> 19;       // 13 bits
@@ -204,7 +207,7 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
   // neighbour table in list positions, and the 32-row blocks' offset masks
   unsigned long long mine = 0;
   for (int k = 0; k < k_vol; ++k) {
-    const int g = row >= 0 ? nbr[(size_t)k * n_dst + row] : -1;
+    const int g = row >= 0 ? nbr[(size_t)k * n_dst + col] : -1;
     unsigned short lid = kNoNbr;
     if (g >= 0) {
       const int key = inv_src ? inv_src[g] : g;
@@ -543,10 +546,10 @@ int halo_morton_order(const int32_t *coords, int64_t n, int coord_bits, int32_t 
 }
 
 // Builds direction d of the plan's tile tables (0: forward, destination = output rows;
-// 1: input gradient, destination = input rows) from the neighbour table by destination row.
+// 1: input gradient, destination = input rows) from the plan's neighbour table.
 // flags: two device ints, zeroed by the caller (see halo_build_kernel).
-int halo_build(Plan *p, int d, const int32_t *nbr_by_row, const int32_t *order_dst, const int32_t *inv_src,
-               const int32_t *order_src, int *flags, hipStream_t s) {
+int halo_build(Plan *p, int d, const int32_t *nbr_by_pos, const int32_t *plan_pos, const int32_t *order_dst,
+               const int32_t *inv_src, const int32_t *order_src, int *flags, hipStream_t s) {
   HaloSide &hs = p->halo[d];
   hs = HaloSide{};
   const int64_t n_dst = d ? p->n_in : p->n_out;
@@ -564,7 +567,7 @@ int halo_build(Plan *p, int d, const int32_t *nbr_by_row, const int32_t *order_d
     return FGMS_E_NOMEM;
   }
   halo_build_kernel<<<(unsigned)hs.n_tiles, kBuildThreads, 0, s>>>(
-      nbr_by_row, order_dst, inv_src, order_src, (int)n_dst, p->k_vol, sort_by_mask, hs.list_cap, hs.order,
+      nbr_by_pos, plan_pos, order_dst, inv_src, order_src, (int)n_dst, p->k_vol, sort_by_mask, hs.list_cap, hs.order,
       hs.rows, hs.count, hs.lnbr, hs.mask32, flags);
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;

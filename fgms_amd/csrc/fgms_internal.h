@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <vector>
 
 #include "../../include/fgms.h"
@@ -107,9 +108,21 @@ struct HaloSide {
   bool ok;                      // built and every tile's list fitted list_cap
 };
 
+constexpr int kPlanFlags = 13;      // ints the plan build reports back (see fgms_plan.hip)
+
 // Plan: neighbour tables built from the pair lists.
 struct Plan {
   int device;
+  // the build is asynchronous: `flags` (device) is copied to `host_flags` (pinned) behind the
+  // build's last kernel, `ready` fires after that copy; plan_resolve reads them on first use
+  int *flags;
+  int *host_flags;
+  hipEvent_t ready;
+  std::mutex mutex;
+  bool resolved, invalid;
+  bool has_tables;        // k_vol <= 64: neighbour tables and masks exist (else the plan is the weight gradient's bands only)
+  const int32_t *kpos, *in_map, *out_map;    // the caller's lists (for the pair view, built on first use)
+  hipStream_t pv_stream;
   int k_vol;
   int64_t n_in, n_out, n_pairs;
   // Destination rows are visited in a plan-chosen order (rows with the same set
@@ -145,6 +158,12 @@ struct Plan {
   int32_t *tile_out, *tile_in;
   int tile_grid_out, tile_grid_in;   // entries of the tables (a multiple of 8)
   mutable hipStream_t last_stream;   // the stream of the latest launch that read the plan
+  mutable bool many_streams;         // launches on more than one stream have read it (destroy then drains the device)
+  // a transposed view (fgms_plan_transposed) shares the tables of `base` with the sides swapped
+  // and owns nothing; `views` counts the views alive on a base, which is freed after the last one
+  Plan *base;
+  int views;
+  bool destroyed;
   // (64-row block, offset) combinations with at least one pair: the output-stationary
   // kernels run stages * 64 row slots for n_pairs pairs
   int stages_out, stages_in;
@@ -214,8 +233,15 @@ int launch_pair_view_gms(const GmsArgs &a, const Plan *p);
 // Tile tables of the LDS-neighbourhood kernels (fgms_halo.hip).
 int halo_morton_order(const int32_t *coords, int64_t n, int coord_bits, int32_t **order, int32_t **inv,
                       std::vector<void *> *tmp, hipStream_t s);
-int halo_build(Plan *p, int d, const int32_t *nbr_by_row, const int32_t *order_dst, const int32_t *inv_src,
-               const int32_t *order_src, int *flags, hipStream_t s);
+int halo_build(Plan *p, int d, const int32_t *nbr_by_pos, const int32_t *plan_pos, const int32_t *order_dst,
+               const int32_t *inv_src, const int32_t *order_src, int *flags, hipStream_t s);
+// Notes that a launch on `stream` reads the plan.
+inline void plan_touch(const Plan *p, hipStream_t stream) {
+  if (p->last_stream != stream && p->resolved) p->many_streams = true;
+  p->last_stream = stream;
+}
+// The plan with its build results known, or nullptr (see fgms_plan.hip).
+const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc);
 void halo_release(Plan *p);
 bool halo_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_halo_gms(const GmsArgs &a, const Plan *p);

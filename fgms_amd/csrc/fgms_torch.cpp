@@ -6,9 +6,13 @@
 //  * work is queued on torch's current HIP stream, not on stream 0
 //    (the reference uses bare <<<>>> launches, backend/spconv.cu:112);
 //  * a kernel-map plan is built on first use of a (kpos, in_map, out_map)
-//    triple and kept in a small cache; an entry holds references to the three
-//    tensors, so their storage cannot be recycled while it is cached, and is
-//    dropped when one of them is modified in place (version counter);
+//    triple (asynchronously: the call queues the build and goes on) and kept in a
+//    small cache; an entry holds references to the three tensors, so their storage
+//    cannot be recycled while it is cached, and is dropped when one of them is
+//    modified in place (version counter; writes through raw pointers do not bump
+//    it, and tensors made under inference mode have none: clear the cache after
+//    rewriting such a map).  A call with in_map and out_map exchanged (the
+//    transposed convolution over the same pairs) shares the cached plan's tables;
 //  * HIP errors raise RuntimeError instead of passing silently.
 #include <torch/extension.h>
 
@@ -30,7 +34,13 @@ struct CacheEntry {
   int64_t n_in, n_out;
   int device;
   fgms_plan_t *plan;
+  bool view;                              // a transposed view of another entry's plan
 };
+
+// Inference tensors track no version.
+int64_t version_of(const at::Tensor &t) { return t.is_inference() ? 0 : (int64_t)t._version(); }
+
+size_t g_views_made = 0;
 
 std::mutex g_mutex;
 std::list<CacheEntry> g_cache;            // most recently used first
@@ -92,8 +102,8 @@ fgms_plan_t *plan_for(const at::Tensor &kpos, const at::Tensor &in_map, const at
   for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
     if (it->in_map.is_same(in_map) && it->out_map.is_same(out_map) && it->kpos.is_same(kpos) &&
         it->n_in == n_in && it->n_out == n_out && it->device == dev) {
-      if (it->v_in == in_map._version() && it->v_out == out_map._version() &&
-          it->v_kpos == kpos._version()) {
+      if (it->v_in == version_of(in_map) && it->v_out == version_of(out_map) &&
+          it->v_kpos == version_of(kpos)) {
         g_cache.splice(g_cache.begin(), g_cache, it);
         return g_cache.front().plan;
       }
@@ -101,11 +111,30 @@ fgms_plan_t *plan_for(const at::Tensor &kpos, const at::Tensor &in_map, const at
       break;
     }
   }
+  // a map first seen while the stream is being captured into a graph: no plan is built (the build
+  // allocates, and its kernels would be recorded); the call records the kernels that need none
+  {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone) return nullptr;
+  }
   fgms_plan_t *plan = nullptr;
-  check(fgms_plan_create(&plan, i32(kpos), i32(in_map), i32(out_map), n_in, n_out, k_vol,
-                         in_map.numel(), stream));
-  g_cache.push_front(CacheEntry{kpos, in_map, out_map, kpos._version(), in_map._version(),
-                                out_map._version(), n_in, n_out, dev, plan});
+  bool view = false;
+  // the same pairs with the sides exchanged: share that plan's tables
+  for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
+    if (!it->view && it->in_map.is_same(out_map) && it->out_map.is_same(in_map) && it->kpos.is_same(kpos) &&
+        it->n_in == n_out && it->n_out == n_in && it->device == dev && it->v_in == version_of(out_map) &&
+        it->v_out == version_of(in_map) && it->v_kpos == version_of(kpos)) {
+      check(fgms_plan_transposed(&plan, it->plan));
+      view = true;
+      ++g_views_made;
+      break;
+    }
+  }
+  if (!plan)
+    check(fgms_plan_create(&plan, i32(kpos), i32(in_map), i32(out_map), n_in, n_out, k_vol,
+                           in_map.numel(), stream));
+  g_cache.push_front(CacheEntry{kpos, in_map, out_map, version_of(kpos), version_of(in_map),
+                                version_of(out_map), n_in, n_out, dev, plan, view});
   while (g_cache.size() > g_cache_cap) drop(std::prev(g_cache.end()));
   return plan;
 }
@@ -193,6 +222,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("fgms_plan_cache", &set_cache, pybind11::arg("enabled"), pybind11::arg("capacity") = 8);
   m.def("fgms_plan_cache_clear", &clear_cache);
   m.def("fgms_plan_cache_size", &cache_size);
+  m.def("fgms_plan_cache_views", []() { std::lock_guard<std::mutex> lock(g_mutex); return g_views_made; });
   m.def("fgms_version", []() { return std::string(fgms_version()); });
   m.def("fgms_set_kernel_policy", &fgms_set_kernel_policy);
 }

@@ -539,7 +539,7 @@ int wgrad_static(WgradArgs a) {
   }
   a.side = SideJob{};
   a.deferred_flush = nullptr;
-  if (a.plan) a.plan->last_stream = a.stream;
+  if (a.plan) plan_touch(a.plan, a.stream);
   return launch_mfma_wgrad(a);
 }
 

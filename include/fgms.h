@@ -90,6 +90,14 @@ int fgms_plan_create_coords(fgms_plan_t **plan, const int32_t *kpos,
                             int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
                             const int32_t *in_coords, const int32_t *out_coords,
                             int coord_bits, void *stream);
+/*
+ * A plan for the same pairs with the roles of the two sides swapped (in_map and out_map
+ * exchanged: the map of the transposed convolution, backend/spconv.cu:460 swaps them the
+ * same way for the input gradient).  It shares the tables of `base`, which already hold both
+ * directions, and costs nothing to make; destroy it like any plan (the shared tables go with
+ * the last of base and its views).  No counterpart in the reference.
+ */
+int fgms_plan_transposed(fgms_plan_t **view, fgms_plan_t *base);
 void fgms_plan_destroy(fgms_plan_t *plan);
 /* 1 if the output-stationary kernels can use it for forward / for dgrad. */
 int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad);

@@ -206,8 +206,18 @@ def test_out_of_range_map_is_rejected_by_plan(capi):
     kpos = torch.tensor([0, 2, 4], dtype=torch.int32, device="cuda")
     imap = torch.tensor([0, 1, 2, 99], dtype=torch.int32, device="cuda")
     omap = torch.tensor([0, 1, 2, 3], dtype=torch.int32, device="cuda")
+    # the build is asynchronous: the plan is handed out at once, what the build found is
+    # known (and reported) when the plan is first asked about or used
+    plan = capi.Plan(kpos, imap, omap, 10, 10)
+    assert not plan.usable() and not plan.usable(for_dgrad=True)
+    x = torch.zeros(10, 32, device="cuda")
+    w = torch.zeros(2, 32, 32, device="cuda")
+    out = torch.zeros(10, 32, device="cuda")
     with pytest.raises(ValueError, match="outside"):
-        capi.Plan(kpos, imap, omap, 10, 10)
+        capi.fusion_fwd(x, w, 0, out, kpos, None, imap, omap, False, False, plan=plan)
+    with pytest.raises(ValueError, match="outside"):
+        plan.stats()
+    plan.close()
 
 
 def test_empty_inputs(capi):

@@ -1,0 +1,138 @@
+"""The plan as an object: asynchronous build, transposed views that share a plan's tables,
+the python extension's cache recognising a swapped map, HIP-graph capture that includes the
+first call on a map, tensors made under inference mode."""
+import numpy as np
+import pytest
+import torch
+
+from fgms_amd import clouds
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from fgms_amd import capi as c
+    c.lib()
+    assert torch.cuda.is_available()
+    yield c
+    c.set_kernel_policy(0)
+
+
+def strided_layers(dtype=np.float16, n=20000, c_in=64, c_out=128):
+    rng = np.random.default_rng(31)
+    vin = clouds.cloud_indoor(clouds.rng_for(2), target=n)
+    vout = clouds.downsample_coords(vin, 2)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vin, vout, clouds.offsets_cube(2), stride=2)
+    down = clouds.make_layer(rng, imap, omap, knnz, kpos, len(vin), len(vout), c_in, c_out, dtype)
+    up = clouds.make_layer(rng, omap, imap, knnz, kpos, len(vout), len(vin), c_out, c_in, dtype)
+    return down, up
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32], ids=["fp16", "fp32"])
+def test_transposed_view_shares_the_tables(capi, oracle, dtype):
+    """The transposed convolution's map is the same pairs with the sides exchanged: a view of
+    the down-sampling layer's plan serves the up-sampling layer, all three passes."""
+    down, up = strided_layers(dtype)
+    Dd, Du = G.to_dev(down), G.to_dev(up)
+    mode = G.mode_of(dtype)
+    plan = capi.Plan(Dd["kpos"], Dd["imap"], Dd["omap"], Dd["n_in"], Dd["n_out"])
+    view = plan.transposed()
+    assert view.usable() == plan.usable(for_dgrad=True) and view.usable(for_dgrad=True) == plan.usable()
+    sv, sp = view.stats(), plan.stats()
+    assert sv["pairs"] == sp["pairs"] and sv["blocks_fwd"] == sp["blocks_dgrad"] and sv["blocks_dgrad"] == sp["blocks_fwd"]
+    a = (up["knnz"], up["imap"], up["omap"])
+    capi.profile_reset(); capi.profile_enable(True)
+    out = G.run_fwd(capi, Du, plan=view)
+    gi, gw = G.run_bwd(capi, Du, plan=view)
+    capi.profile_enable(False)
+    names = {n for n, _ in capi.profile_records()}
+    capi.profile_reset()
+    assert any(n.startswith(("gms_rows_kernel", "bwd_fused_kernel")) for n in names), names
+    G.assert_close(out, oracle.c_fwd(up["in_feats"], up["kernel"], *a, up["n_out"]), mode, "fwd through the view")
+    G.assert_close(gi, oracle.c_dgrad(up["out_grad"], up["kernel"], *a, up["n_in"]), mode, "dgrad through the view")
+    G.assert_close(gw, oracle.np_wgrad(up["in_feats"], up["out_grad"], *a, up["k_vol"]), mode, "wgrad through the view")
+    # the base can go first: the tables live until the last view does
+    plan.close()
+    out2 = G.run_fwd(capi, Du, plan=view)
+    assert np.array_equal(out, out2)
+    view.close()
+
+
+def test_backend_cache_shares_a_swapped_map(oracle):
+    import FGMS.backend as B
+    import FGMS.nn as fnn
+    down, up = strided_layers()
+    Dd = G.to_dev(down)
+    B.fgms_plan_cache_clear()
+    made = B.fgms_plan_cache_views()
+    kmap = fnn.KernelMap(Dd["imap"], Dd["omap"], down["knnz"], Dd["n_in"], Dd["n_out"])
+    x = torch.from_numpy(down["in_feats"]).cuda()
+    wd = torch.from_numpy(down["kernel"]).cuda()
+    wu = torch.from_numpy(up["kernel"]).cuda()
+    y = fnn.sparse_conv(x, wd, kmap)
+    z = fnn.sparse_conv(y, wu, kmap.transposed())
+    torch.cuda.synchronize()
+    assert B.fgms_plan_cache_size() == 2 and B.fgms_plan_cache_views() == made + 1
+    a = (down["knnz"], down["imap"], down["omap"])
+    y_ref = oracle.c_fwd(down["in_feats"], down["kernel"], *a, down["n_out"])
+    G.assert_close(y.cpu().numpy(), y_ref, "fp16", "down")
+    z_ref = oracle.c_fwd(y.cpu().numpy(), up["kernel"], up["knnz"], up["imap"], up["omap"], up["n_out"])
+    G.assert_close(z.cpu().numpy(), z_ref, "fp16", "up through the shared plan")
+    B.fgms_plan_cache_clear()
+
+
+def test_first_call_on_a_map_inside_a_captured_graph(oracle):
+    """fgms_plan_create queues the build and returns; a call recorded into a HIP graph right
+    behind it cannot wait for the build's findings, so it records the kernels that need no
+    plan.  Every replay must give the oracle's result; calls after the capture use the plan."""
+    import FGMS.backend as B
+    rng = np.random.default_rng(8)
+    vox = clouds.dedup(clouds._sphere_shell(rng, np.array([10., 10, 10]), 7.0, 6000), 20)
+    L = clouds.submanifold_case(vox, 64, 64, np.float16, rng)
+    D = G.to_dev(L)
+    out = torch.zeros(L["n_out"], 64, dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
+    other = clouds.submanifold_case(vox[:2000], 64, 64, np.float16, rng)
+    Do = G.to_dev(other)
+    oo = torch.zeros(other["n_out"], 64, dtype=torch.float16, device="cuda")
+    with torch.cuda.stream(side):      # workspaces of this shape exist before the capture (another map)
+        B.fgms_fusion_fwd_cuda(Do["in_feats"], Do["kernel"], 0, oo, Do["kpos"], Do["kpos"], Do["imap"], Do["omap"], False, False)
+        B.fgms_plan_cache(False)
+        B.fgms_fusion_fwd_cuda(Do["in_feats"], Do["kernel"], 0, oo, Do["kpos"], Do["kpos"], Do["imap"], Do["omap"], False, False)
+        B.fgms_plan_cache(True)
+    torch.cuda.synchronize()
+    want = oracle.c_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side, capture_error_mode="thread_local"):
+        out.zero_()
+        B.fgms_fusion_fwd_cuda(D["in_feats"], D["kernel"], 0, out, D["kpos"], D["kpos"], D["imap"], D["omap"], False, False)
+    for _ in range(3):
+        out.fill_(3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        G.assert_close(out.cpu().numpy(), want, "fp16", "replay")
+    out.zero_()
+    B.fgms_fusion_fwd_cuda(D["in_feats"], D["kernel"], 0, out, D["kpos"], D["kpos"], D["imap"], D["omap"], False, False)
+    torch.cuda.synchronize()
+    G.assert_close(out.cpu().numpy(), want, "fp16", "eager call after the capture")
+    B.fgms_plan_cache_clear()
+
+
+def test_inference_mode_tensors(oracle):
+    import FGMS.backend as B
+    rng = np.random.default_rng(9)
+    vox = clouds.cloud_indoor(clouds.rng_for(2), target=3000)
+    L = clouds.submanifold_case(vox, 32, 32, np.float32, rng)
+    with torch.inference_mode():
+        D = G.to_dev(L)
+        out = torch.zeros(L["n_out"], 32, device="cuda")
+        for _ in range(2):          # the second call finds the plan in the cache
+            out.zero_()
+            B.fgms_fusion_fwd_cuda(D["in_feats"], D["kernel"], 0, out, D["kpos"], D["kpos"], D["imap"], D["omap"], False, False)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+    G.assert_close(got, oracle.c_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"]), "fp32", "fwd")
+    B.fgms_plan_cache_clear()
