@@ -106,7 +106,20 @@ def build_cabi_demo(verbose=False):
     return DEMO_PATH
 
 
-def build_all(verbose=False):
+def up_to_date():
+    """True when both shared objects exist and are newer than every source and header."""
+    outs = [LIB_PATH, torch_ext_path()]
+    if not all(os.path.exists(o) for o in outs):
+        return False
+    srcs = [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + \
+           [os.path.join(ROOT, "include", f) for f in os.listdir(os.path.join(ROOT, "include"))]
+    return min(os.path.getmtime(o) for o in outs) >= max(os.path.getmtime(f) for f in srcs)
+
+
+def build_all(verbose=False, force=True):
+    """force=False: keep in-tree products that are newer than all sources."""
+    if not force and up_to_date():
+        return
     build_hip_lib(verbose)
     build_torch_ext(verbose)
     build_cabi_demo(verbose)

@@ -86,6 +86,23 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *
   return FGMS_OK;
 }
 
+// ---- dynamic-LDS limits already granted, per (device, kernel) ------------------
+namespace {
+std::mutex g_lds_mutex;
+std::map<std::pair<int, const void *>, size_t> g_lds_granted;
+}  // namespace
+
+int allow_dynamic_lds(const void *kernel, size_t bytes) {
+  int dev = 0;
+  FGMS_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_lds_mutex);
+  size_t &granted = g_lds_granted[{dev, kernel}];
+  if (granted >= bytes) return FGMS_OK;
+  FGMS_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  granted = bytes;
+  return FGMS_OK;
+}
+
 // ---- block pool: device memory of plans and of the map builder's temporaries --
 // hipMalloc / hipFree cost 50-100 us each and a plan needs a dozen blocks, which
 // made building a plan (once per kernel map, i.e. several times per training

@@ -596,12 +596,7 @@ int launch_halo_gms(const GmsArgs &a, const Plan *p) {
   const HaloSide &hs = p->halo[a.transpose_w ? 1 : 0];
   const int c_dst = a.transpose_w ? a.c_in : a.c_out;
   auto kern = a.transpose_w ? gms_halo_kernel<2> : gms_halo_kernel<1>;
-  static bool attr_set[2] = {false, false};
-  if (!attr_set[a.transpose_w ? 1 : 0]) {
-    FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kHaloLds));
-    attr_set[a.transpose_w ? 1 : 0] = true;
-  }
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)kHaloLds); if (rc_lds != FGMS_OK) return rc_lds; }
   const unsigned gx = (unsigned)((hs.n_tiles + 7) / 8 * 8);
   {
     ProfileScope prof(a.transpose_w ? "gms_halo_kernel(dgrad)" : "gms_halo_kernel(fwd)", a.stream);

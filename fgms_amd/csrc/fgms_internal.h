@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "../../include/fgms.h"
+#include "../../include/fgms_diag.h"
 
 namespace fgms {
 
@@ -207,6 +208,9 @@ bool mfma_gms_supported(const GmsArgs &a);
 int pool_alloc(void **ptr, size_t bytes, hipStream_t user);
 void pool_free(void *ptr, hipStream_t last_user, bool idle);
 void pool_trim(size_t keep_bytes);
+// Raises a kernel's dynamic-LDS limit to `bytes` (hipFuncSetAttribute) unless an earlier call
+// on this device already allowed as much: the attribute call costs a microsecond per launch.
+int allow_dynamic_lds(const void *kernel, size_t bytes);
 int kernel_policy();   // fgms_set_kernel_policy's value
 int num_cus();         // compute units of the current device
 int launch_mfma_gms(const GmsArgs &a);

@@ -746,8 +746,7 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   const int tiles_per_wg = (int)((tiles + want_wgs - 1) / want_wgs);
   const unsigned gx = (unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg);
   auto kern = split ? gms_pairs_kernel<T, NT, S, kCanSplit> : gms_pairs_kernel<T, NT, S, false>;
-  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)s.lds_bytes));
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)s.lds_bytes); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof(split ? (a.transpose_w ? "gms_pairs_kernel(dgrad, bf16x3)" : "gms_pairs_kernel(fwd, bf16x3)")
                             : (a.transpose_w ? "gms_pairs_kernel(dgrad)" : "gms_pairs_kernel(fwd)"),
@@ -810,9 +809,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
               : raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0>
               : raw == 1 ? gms_rows_kernel<T, NT, S, kCanRaw && sizeof(T) == 2 ? 1 : 0>
                          : gms_rows_kernel<T, NT, S, 0>;
-  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)s.lds_rows_bytes));
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)s.lds_rows_bytes); if (rc_lds != FGMS_OK) return rc_lds; }
   // A launch that fills less than half of the chip's workgroup slots shares every
   // tile between two workgroups, each taking half of the tile's offsets and adding
   // its part with atomics: twice the workgroups, half the critical path.  (Two
@@ -907,8 +904,7 @@ int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArg
   constexpr bool kCanSplit = sizeof(T) == 4 && S == 4 && NT != 4;
   const bool split = kCanSplit && d.reduced && split_bf16_enabled() && g.split;
   auto kern = split ? bwd_fused_kernel<T, NT, S, BI, BJ, kCanSplit ? 4 : 2> : bwd_fused_kernel<T, NT, S, BI, BJ, 2>;
-  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)lds); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof(split ? "bwd_fused_kernel(bf16x3)" : "bwd_fused_kernel", d.stream);
     kern<<<row_x * row_y * row_z + (unsigned)(g.tiles * g.ty), kThreads, lds, d.stream>>>(

@@ -25,6 +25,7 @@
 #include <stdexcept>
 
 #include "fgms.h"
+#include "fgms_diag.h"
 
 namespace {
 

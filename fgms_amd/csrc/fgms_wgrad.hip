@@ -283,8 +283,7 @@ int launch(const WgradArgs &a, float *acc32) {
   if (rc != FGMS_OK) return rc;
   constexpr bool kCanSplit = sizeof(T) == 4;
   auto kern = g.split ? wgrad_kernel<T, BI, BJ, kCanSplit> : wgrad_kernel<T, BI, BJ, false>;
-  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds));
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)g.lds); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof(g.split ? "wgrad_kernel(bf16x3)" : "wgrad_kernel", a.stream);
     kern<<<dim3((unsigned)g.tiles + (unsigned)a.side.blocks, (unsigned)g.ty), kThreads, g.lds, a.stream>>>(
@@ -302,8 +301,7 @@ int launch_wave(const WgradArgs &a, float *acc32) {
   if (rc != FGMS_OK) return rc;
   constexpr bool kCanSplit = sizeof(T) == 4;
   auto kern = g.split ? wgrad_wave_kernel<T, BI, BJ, kCanSplit> : wgrad_wave_kernel<T, BI, BJ, false>;
-  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds));
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)g.lds); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof(g.split ? "wgrad_wave_kernel(bf16x3)" : "wgrad_wave_kernel", a.stream);
     kern<<<dim3((unsigned)g.tiles + (unsigned)a.side.blocks, (unsigned)g.ty), kThreads, g.lds, a.stream>>>(
@@ -337,8 +335,7 @@ int launch_skinny(const WgradArgs &a, float *acc32) {
   const int64_t tiles = (int64_t)smap.slices * a.k_vol;
   const size_t lds = (size_t)(kSkinnyThreads / 64 - 1) * CS * CD * sizeof(float);
   auto kern = wgrad_skinny_kernel<T, CS, CD>;
-  FGMS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)lds); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof("wgrad_skinny_kernel", a.stream);
     kern<<<(unsigned)tiles, kSkinnyThreads, lds, a.stream>>>(

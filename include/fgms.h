@@ -63,11 +63,19 @@ const char *fgms_last_error(void);
 /*
  * Kernel-map plan.  Built once per (in_map, out_map, kpos) on the device and
  * reusable by every layer and every pass that shares the map: a neighbour
- * table "output row x offset -> input row" (and its transpose for dgrad).  The
- * reference has no counterpart: it re-reads the pair lists on every call
- * (backend/spconv.cuh:457-563).  Creation synchronises `stream` once to learn
- * whether some offset maps two pairs onto one output row (then the plan is
- * marked non-functional and the entry points silently use the atomic kernels).
+ * table "output row x offset -> input row" (and its transpose for dgrad), the rows
+ * of each side ordered by the set of offsets they use.  The reference has no
+ * counterpart: it re-reads the pair lists on every call (backend/spconv.cuh:457-563).
+ * The build is QUEUED on `stream` and the call returns without waiting for it, like every
+ * other entry point.  What the build finds out about the map -- an index outside
+ * [0, n_in) x [0, n_out), an offset that maps two pairs onto one row (the plan is then
+ * not usable for that direction and the entry points silently use the atomic
+ * kernels), pair order, block counts -- is read when the plan is first used or asked
+ * about: that call waits for the build if it has not finished, and an entry point
+ * given a plan whose map has an out-of-range index returns FGMS_E_INVALID.  Exception:
+ * a first use recorded into a HIP graph (stream capture) cannot wait and records the
+ * kernels that need no plan.  The map arrays must stay valid and unchanged while the plan
+ * lives.  Not to be called on a stream that is being captured.
  */
 int fgms_plan_create(fgms_plan_t **plan, const int32_t *kpos,
                      const int32_t *in_map, const int32_t *out_map,
@@ -188,25 +196,6 @@ int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *ke
                       int64_t n_in, int64_t n_out, int c_in, int c_out, int k_vol,
                       int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
 
-/* Selects kernels by hand for tests and profiling: 0 = automatic dispatch,
- * 1 = force the generic (non-MFMA) kernels, 2 = force the pair-stationary MFMA
- * kernels even when a usable plan is passed, 3 = automatic dispatch but the
- * output-stationary kernel uses its 128-column wave tiles whenever the layer
- * has a multiple of 128 output channels (normally only large fp16 layers),
- * 4 = automatic dispatch but never the pair-stationary kernel where the
- * output-stationary one can run: forward and input-gradient results are then the
- * same bit for bit from run to run (automatic dispatch gives wide layers over
- * scattered clouds, with few pairs per 64-row block and offset, to the
- * pair-stationary kernel, whose atomic sums depend on their order; fp32 layers of
- * that kind run the output-stationary kernel's body over the plan's pair view, also
- * with atomic sums),
- * 5 = forward and input gradient over the plan's pair view whenever the plan has
- * one (plans created under this policy keep it for dense maps too),
- * 6 = forward and input gradient of fp16 layers with 64 source channels through the kernel
- * that keeps a tile's neighbourhood rows in LDS, for plans made by fgms_plan_create_coords.
- * Process-wide. */
-void fgms_set_kernel_policy(int policy);
-
 /*
  * Kernel-map builder.  No counterpart in the reference, whose scripts load the
  * maps from files (cpu-check.py:89-94, spconv-test.py:64-73); this is the step
@@ -228,32 +217,6 @@ int fgms_build_kernel_map(const int32_t *in_coords, int64_t n_in,
                           const int32_t *offsets, int k_vol, int stride, int skip_offset,
                           int32_t *in_map, int32_t *out_map, int64_t capacity,
                           int32_t *kernel_nnz, int32_t *kpos, int64_t *n_pairs, void *stream);
-
-/*
- * Diagnostic, no counterpart in the reference: reads exactly the feature rows
- * the output-stationary forward (for_dgrad = 0: feats = in_feats, c_src = c_in)
- * or input-gradient kernel (for_dgrad != 0: feats = out_feats_grad,
- * c_src = c_out) gathers for this plan, and nothing else: no weights, no
- * matrix cores, no result.  Timed through fgms_profile_* it gives the time the
- * memory system alone needs for the gathers of one pass, the floor that the
- * real kernel's duration is compared with.  Rows must be 16 * 2^j bytes
- * (j = 0..6); k_vol <= 64.
- */
-int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad,
-                      fgms_plan_t *plan, void *stream);
-
-/*
- * Per-kernel timing with HIP events on the stream the kernels are launched on
- * (no counterpart in the reference, which times whole calls from python,
- * spconv-test.py:95-122).  While enabled, every main kernel launch (not the
- * small weight re-layout or zero-fill launches) is bracketed by two events.
- * fgms_profile_read synchronises with the recorded events and returns the
- * index-th record: kernel name and milliseconds; it returns FGMS_E_INVALID
- * once index runs past the records.  fgms_profile_reset drops all records.
- */
-void fgms_profile_enable(int on);
-int fgms_profile_read(int index, char *name, int name_len, float *ms);
-void fgms_profile_reset(void);
 
 #ifdef __cplusplus
 }

@@ -1,6 +1,7 @@
 """The C-ABI library loads on a machine without a GPU and exports every symbol
-that include/fgms.h declares; the python extension keeps the reference's three
-function names (backend/pybind_cuda.cpp:8-10)."""
+that include/fgms.h (the drop-in surface) and include/fgms_diag.h (tests and
+measurement) declare; the python extension keeps the reference's three function
+names (backend/pybind_cuda.cpp:8-10)."""
 import ctypes
 import os
 import re
@@ -10,16 +11,22 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "fgms.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(fgms_[a-z0-9_]+)\s*\(", text)))
+def declared_symbols(headers=("fgms.h", "fgms_diag.h")):
+    found = set()
+    for h in headers:
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        found |= set(re.findall(r"\b(fgms_[a-z0-9_]+)\s*\(", text))
+    return sorted(found)
 
 
 def test_header_declares_the_reference_entry_points():
-    syms = declared_symbols()
+    syms = declared_symbols(("fgms.h",))
     for s in ("fgms_fusion_fwd", "fgms_fwd", "fgms_bwd"):
         assert s in syms
+    # the drop-in header carries no test or measurement entry points
+    for s in syms:
+        assert not s.startswith(("fgms_profile", "fgms_probe", "fgms_set_kernel_policy")), s
 
 
 def test_library_exports_every_declared_symbol():
