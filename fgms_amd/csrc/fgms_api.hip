@@ -283,8 +283,8 @@ int check_common(const void *a, const void *b, const void *c, const int32_t *kpo
 // The kernel without atomics, whose results do not depend on the run, gets 5 % on top.
 bool sparse_rows(const GmsArgs &a, const Plan *plan) {
   const int stages = a.transpose_w ? plan->stages_in : plan->stages_out;
-  if (stages <= 0 || plan->n_pairs <= 0) return false;   // (the plan's own pair count: a.n_pairs is a bound)
-  const double slots_per_pair = (double)stages * 64.0 / (double)plan->n_pairs;
+  if (stages <= 0 || plan->pairs_counted <= 0) return false;   // (the plan's own pair count: a.n_pairs is a bound)
+  const double slots_per_pair = (double)stages * 64.0 / (double)plan->pairs_counted;
   const double c_src = a.transpose_w ? a.c_out : a.c_in;
   const double even = a.dtype == FGMS_F16 ? 2.2 + 16.0 / c_src : 1.0 + 45.0 / c_src;
   // (no break-even point was measured below 1.3: denser maps stay output-stationary)
@@ -317,7 +317,28 @@ Route route_of(const GmsArgs &a, const Plan *plan) {
   return mfma_gms_supported(a) ? Route::kPairs : Route::kGeneric;
 }
 
+int run_gms_one(GmsArgs a, const Plan *plan);
+
+// A pass over all offsets: one walk for plans of up to 64 offsets (or none), one per group of 64
+// offsets for larger kernels (the groups' results add up in the destination rows).
 int run_gms(GmsArgs a, const Plan *plan) {
+  if (!plan || plan->groups.empty() || a.dense_k >= 0) return run_gms_one(a, plan);
+  plan_touch(plan, a.stream);
+  const size_t esz = a.dtype == FGMS_F16 ? 2 : 4;
+  int k0 = 0;
+  for (const Plan *g : plan->groups) {
+    GmsArgs ga = a;
+    ga.w = (const char *)a.w + (size_t)k0 * a.c_in * a.c_out * esz;
+    ga.kpos = a.kpos + k0;
+    ga.k_vol = g->k_vol;
+    int rc = run_gms_one(ga, g);
+    if (rc != FGMS_OK) return rc;
+    k0 += g->k_vol;
+  }
+  return FGMS_OK;
+}
+
+int run_gms_one(GmsArgs a, const Plan *plan) {
   if (plan) plan_touch(plan, a.stream);
   const bool dense = a.dense_k >= 0;
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
@@ -553,7 +574,7 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
   // gradient goes first and its launch also re-lays the weights for the input gradient,
   // whose launch in turn also rounds the weight gradient's fp32 sums into the caller's
   // fp16 tensor.  (The two gradients do not depend on each other.)
-  if (n_pairs > 0 && route_of(d, p) == Route::kRows && g_policy != 1 && mfma_wgrad_supported(w)) {
+  if (n_pairs > 0 && (!p || p->groups.empty()) && route_of(d, p) == Route::kRows && g_policy != 1 && mfma_wgrad_supported(w)) {
     plan_touch(p, d.stream);
     // one launch for both where the shapes allow (and a small one that rounds an fp16
     // weight gradient), else two

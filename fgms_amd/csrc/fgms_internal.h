@@ -121,6 +121,10 @@ struct Plan {
   hipEvent_t ready;
   std::mutex mutex;
   bool resolved, invalid;
+  bool has_bands;         // the weight gradient's row-band tables were built
+  bool ordered;           // every offset's pairs are ordered by output row (what the bands need)
+  int64_t pairs_counted;  // pairs the build saw (kpos[k_vol] - kpos[0]); n_pairs is the caller's bound
+  std::vector<Plan *> groups;   // k_vol > 64: one plan per 64 offsets (owned)
   bool has_tables;        // k_vol <= 64: neighbour tables and masks exist (else the plan is the weight gradient's bands only)
   const int32_t *kpos, *in_map, *out_map;    // the caller's lists (for the pair view, built on first use)
   hipStream_t pv_stream;

@@ -45,7 +45,7 @@ __global__ void pair_masks_kernel(const int32_t *__restrict__ kpos, const int32_
                                   int n_out, unsigned long long *__restrict__ rmask_out,
                                   unsigned long long *__restrict__ rmask_in, int *__restrict__ flags) {
   const int total = kpos[k_vol];
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  const int j = kpos[0] + blockIdx.x * blockDim.x + threadIdx.x;      // (kpos[0] > 0: a plan over a slice of the offsets)
   if (j >= total || j >= n_pairs) return;
   int lo = 0, hi = k_vol;          // offset of pair j: the last k with kpos[k] <= j
   while (hi - lo > 1) {
@@ -54,7 +54,7 @@ __global__ void pair_masks_kernel(const int32_t *__restrict__ kpos, const int32_
   }
   const int k = lo;
   const int i = imap[j], o = omap[j];
-  if (j == 0) flags[12] = min(total, n_pairs);
+  if (j == kpos[0]) flags[12] = min(total, n_pairs) - kpos[0];
   if (i < 0 || i >= n_in || o < 0 || o >= n_out) {
     flags[0] = 1;
     return;
@@ -272,7 +272,7 @@ __global__ void tables_kernel(const int32_t *__restrict__ kpos, const int32_t *_
                               const int32_t *__restrict__ inv_in, int32_t *__restrict__ nbr_out,
                               int32_t *__restrict__ nbr_in) {
   const int total = kpos[k_vol];
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  const int j = kpos[0] + blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= total || j >= n_pairs) return;
   int lo = 0, hi = k_vol;
   while (hi - lo > 1) {
@@ -353,7 +353,7 @@ __global__ void pair_view_kernel(const int32_t *__restrict__ kpos, const int32_t
     vp[k_vol] = v;
   }
   __syncthreads();
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  const int j = kp[0] + blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= kp[k_vol] || j >= n_pairs) return;
   int lo = 0, hi = k_vol;
   while (hi - lo > 1) {
@@ -604,7 +604,8 @@ namespace fgms {
 // plan_resolve when the plan is first used.
 int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
                 const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
-                const int32_t *in_coords, const int32_t *out_coords, int coord_bits, void *stream) {
+                const int32_t *in_coords, const int32_t *out_coords, int coord_bits, void *stream,
+                bool want_bands) {
   if (!plan_out) {
     set_error("plan output pointer is null");
     return FGMS_E_INVALID;
@@ -665,8 +666,8 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   const size_t so = tables ? (size_t)n_out * k_vol : 0, si = tables ? (size_t)n_in * k_vol : 0;
   const size_t bo = (size_t)(n_out + 63) / 64, bi = (size_t)(n_in + 63) / 64;
   unsigned long long *rmask = nullptr;          // [n_out] then [n_in]
-  if (!take((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), false) ||
-      !take((void **)&p->band_cells, (size_t)4 * k_vol * p->band_count * sizeof(int32_t), false) ||
+  if ((want_bands && (!take((void **)&p->band_start, (size_t)k_vol * (p->band_count + 1) * sizeof(int32_t), false) ||
+                      !take((void **)&p->band_cells, (size_t)4 * k_vol * p->band_count * sizeof(int32_t), false))) ||
       !take((void **)&p->flags, kPlanFlags * sizeof(int), false) ||
       (tables && (!take((void **)&p->nbr_out, (so + si) * sizeof(int32_t), false) ||
                   !take((void **)&p->mask_out, (bo + bi) * sizeof(unsigned long long), false) ||
@@ -681,6 +682,7 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   unsigned long long *rmask_out = rmask, *rmask_in = rmask ? rmask + n_out : nullptr;
   if ((rc = fill_i32(p->flags, kPlanFlags, 0, s))) return fail(rc);
   p->has_tables = tables;
+  p->has_bands = want_bands;
 
   // fork: the band tables and the pre-fill of the neighbour tables do not depend on the rest
   static const bool two_streams = !(getenv("FGMS_PLAN_STREAMS") && atoi(getenv("FGMS_PLAN_STREAMS")) == 1);
@@ -703,11 +705,13 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   };
   {
     hipStream_t sb = s2 ? s2 : s;
-    band_bounds_kernel<<<(unsigned)k_vol, 128, 0, sb>>>(kpos, out_map, (int)n_pairs, p->band_count,
-                                                        band_rows > 0 ? band_rows : 1, p->band_start);
-    const int per_xcd = (p->band_count / 8) * k_vol;
-    band_cells_kernel<<<dim3((unsigned)((per_xcd + 255) / 256), 8, 4), 256, 0, sb>>>(
-        p->band_start, k_vol, p->band_count, p->band_cells);
+    if (want_bands) {
+      band_bounds_kernel<<<(unsigned)k_vol, 128, 0, sb>>>(kpos, out_map, (int)n_pairs, p->band_count,
+                                                          band_rows > 0 ? band_rows : 1, p->band_start);
+      const int per_xcd = (p->band_count / 8) * k_vol;
+      band_cells_kernel<<<dim3((unsigned)((per_xcd + 255) / 256), 8, 4), 256, 0, sb>>>(
+          p->band_start, k_vol, p->band_count, p->band_cells);
+    }
     if (tables && (rc = fill_i32(p->nbr_out, so + si, -1, sb))) {
       drop_events();
       return fail(rc);
@@ -849,6 +853,22 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   }
   for (void *q : tmp) pool_free(q, s, false);
   tmp.clear();
+  // More than 64 offsets: the tables and masks hold 64 offsets each, so the offsets are cut
+  // into groups of 64, every group with tables of its own (the pairs of a group are one
+  // contiguous run of the lists); the entry points walk the groups, the weight gradient uses
+  // this plan's row bands over all offsets.
+  if (!tables) {
+    for (int k0 = 0; k0 < k_vol; k0 += 64) {
+      fgms_plan_t *g = nullptr;
+      rc = plan_create(&g, kpos + k0, in_map, out_map, n_in, n_out, k_vol - k0 < 64 ? k_vol - k0 : 64, n_pairs,
+                       in_coords, out_coords, coord_bits, stream, false);
+      if (rc != FGMS_OK) {
+        fgms_plan_destroy((fgms_plan_t *)p);
+        return rc;
+      }
+      p->groups.push_back((Plan *)g);
+    }
+  }
   *plan_out = (fgms_plan_t *)p;
   return FGMS_OK;
 }
@@ -877,6 +897,8 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       p->pv_in = b->pv_out; p->pv_out = b->pv_in; p->pv_mask = b->pv_mask; p->pv_rows = b->pv_rows;
       p->halo[0] = b->halo[1]; p->halo[1] = b->halo[0];
       p->has_tables = b->has_tables;
+      p->pairs_counted = b->pairs_counted;
+      p->ordered = false;
       // (the weight gradient's row bands follow the base's output rows: not valid for the swapped lists)
       p->bands_ok = false; p->band_start = nullptr; p->band_cells = nullptr; p->band_count = 0;
       p->invalid = false;
@@ -901,9 +923,11 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       p->invalid = h[0] != 0;
       p->fwd_ok = p->has_tables && !h[0] && !h[1] && h[10] == h[12];
       p->dgrad_ok = p->has_tables && !h[0] && !h[2] && h[11] == h[12];
-      p->bands_ok = !h[0] && !h[3];
+      p->ordered = !h[0] && !h[3];
+      p->bands_ok = p->has_bands && p->ordered;
       p->stages_out = h[4];
       p->stages_in = h[5];
+      p->pairs_counted = p->has_tables ? h[12] : p->n_pairs;
       for (int d = 0; d < 2; ++d) {
         p->halo[d].ok = p->halo[d].order != nullptr && !h[6 + 2 * d] && !h[0];
         p->halo[d].extra_rounds = h[7 + 2 * d];
@@ -913,12 +937,12 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       // the counts are known, so that dense maps pay nothing.
       static const bool pair_view = !(getenv("FGMS_PAIR_VIEW") && atoi(getenv("FGMS_PAIR_VIEW")) == 0);
       const int most = p->stages_out > p->stages_in ? p->stages_out : p->stages_in;
-      if (!p->invalid && pair_view && p->k_vol <= 64 && p->n_pairs > 0 &&
-          (kernel_policy() == 5 || (double)most * 64.0 >= 1.35 * (double)p->n_pairs)) {
+      if (!p->invalid && pair_view && p->has_tables && p->pairs_counted > 0 &&
+          (kernel_policy() == 5 || (double)most * 64.0 >= 1.35 * (double)p->pairs_counted)) {
         hipStream_t s = stream;
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         const bool capturing = s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
-        const int64_t rows = (p->n_pairs + 64 * (int64_t)p->k_vol + 255) / 256 * 256;
+        const int64_t rows = (p->pairs_counted + 64 * (int64_t)p->k_vol + 255) / 256 * 256;
         if (!capturing &&
             pool_alloc((void **)&p->pv_in, (size_t)rows * sizeof(int32_t), s) == FGMS_OK &&
             pool_alloc((void **)&p->pv_out, (size_t)rows * sizeof(int32_t), s) == FGMS_OK &&
@@ -938,6 +962,21 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
           p->pv_mask = nullptr;
         }
       }
+      // (a plan over more than 64 offsets: its groups)
+      for (Plan *g : p->groups) {
+        int grc = FGMS_OK;
+        const Plan *gr = plan_resolve((fgms_plan_t *)g, stream, &grc);
+        if (!gr && grc == FGMS_E_INVALID) p->invalid = true;
+        if (!gr && grc != FGMS_E_INVALID) return nullptr;        // (cannot be known now: try again later)
+        if (gr) {
+          p->fwd_ok = (g == p->groups.front() ? true : p->fwd_ok) && gr->fwd_ok;
+          p->dgrad_ok = (g == p->groups.front() ? true : p->dgrad_ok) && gr->dgrad_ok;
+          p->stages_out += gr->stages_out;
+          p->stages_in += gr->stages_in;
+          p->ordered = p->ordered && gr->ordered;
+        }
+      }
+      if (!p->groups.empty()) p->bands_ok = p->has_bands && p->ordered && !p->invalid;
       p->resolved = true;
     }
   }
@@ -955,7 +994,7 @@ extern "C" {
 int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
                      const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
                      int64_t n_pairs, void *stream) {
-  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, nullptr, nullptr, 0, stream);
+  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, nullptr, nullptr, 0, stream, true);
 }
 
 int fgms_plan_create_coords(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
@@ -967,13 +1006,13 @@ int fgms_plan_create_coords(fgms_plan_t **plan_out, const int32_t *kpos, const i
     return FGMS_E_INVALID;
   }
   return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, in_coords, out_coords,
-                     coord_bits, stream);
+                     coord_bits, stream, true);
 }
 
 int fgms_plan_transposed(fgms_plan_t **view_out, fgms_plan_t *base_plan) {
   Plan *b = (Plan *)base_plan;
-  if (!view_out || !b || b->base) {
-    set_error("fgms_plan_transposed: needs a plan made by fgms_plan_create");
+  if (!view_out || !b || b->base || !b->groups.empty()) {
+    set_error("fgms_plan_transposed: needs a plan made by fgms_plan_create over at most 64 offsets");
     return FGMS_E_INVALID;
   }
   Plan *v = new Plan();
@@ -1012,6 +1051,12 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
     p->destroyed = true;
     if (p->views > 0) return;       // (still shared: freed with the last view)
   }
+  for (Plan *g : p->groups) {
+    if (p->many_streams) g->many_streams = true;
+    g->last_stream = p->last_stream;
+    fgms_plan_destroy((fgms_plan_t *)g);
+  }
+  p->groups.clear();
   if (p->many_streams) (void)hipDeviceSynchronize();     // (blocks are handed back behind ONE stream's work)
   halo_release(p);
   if (p->nbr_out) pool_free(p->nbr_out, p->last_stream, false);      // (nbr_in is the same block)
@@ -1050,7 +1095,7 @@ int fgms_plan_stats(const fgms_plan_t *plan, int64_t stats[4]) {
   int rc = FGMS_OK;
   const Plan *p = plan_resolve(const_cast<fgms_plan_t *>(plan), nullptr, &rc);
   if (!p) return rc ? rc : FGMS_E_INVALID;
-  stats[0] = p->n_pairs;
+  stats[0] = p->groups.empty() ? p->pairs_counted : p->n_pairs;
   stats[1] = p->stages_out;
   stats[2] = p->stages_in;
   stats[3] = p->pv_in ? p->pv_rows : 0;

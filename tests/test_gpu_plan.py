@@ -136,3 +136,37 @@ def test_inference_mode_tensors(oracle):
         got = out.cpu().numpy()
     G.assert_close(got, oracle.c_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"]), "fp32", "fwd")
     B.fgms_plan_cache_clear()
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32], ids=["fp16", "fp32"])
+def test_more_than_64_offsets_keep_the_output_stationary_kernels(capi, oracle, dtype):
+    """A 5 x 5 x 5 kernel has 125 offsets (the reference takes k_vol from kernel.size(0),
+    backend/spconv.cu:44-45, without a cap): the plan cuts them into groups of 64, each with
+    tables of its own, and forward / input gradient walk the groups with the kernels that
+    need no atomics; the weight gradient uses the plan's row bands over all 125."""
+    rng = np.random.default_rng(41)
+    vox = clouds.cloud_indoor(clouds.rng_for(2), target=6000)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vox, vox, clouds.offsets_cube(5))
+    assert len(knnz) == 125
+    L = clouds.make_layer(rng, imap, omap, knnz, kpos, len(vox), len(vox), 32, 64, dtype)
+    D = G.to_dev(L)
+    mode = G.mode_of(dtype)
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    assert plan.usable() and plan.usable(for_dgrad=True)
+    assert plan.stats()["pairs"] == len(imap)
+    capi.profile_reset(); capi.profile_enable(True)
+    out = G.run_fwd(capi, D, plan=plan)
+    gi, gw = G.run_bwd(capi, D, plan=plan)
+    capi.profile_enable(False)
+    names = [n for n, _ in capi.profile_records()]
+    capi.profile_reset()
+    assert names.count("gms_rows_kernel(fwd)") == 2 and names.count("gms_rows_kernel(dgrad)") == 2, names
+    assert not any("pairs" in n or "generic" in n for n in names), names
+    a = (L["knnz"], L["imap"], L["omap"])
+    G.assert_close(out, oracle.c_fwd(L["in_feats"], L["kernel"], *a, L["n_out"]), mode, "fwd")
+    G.assert_close(gi, oracle.c_dgrad(L["out_grad"], L["kernel"], *a, L["n_in"]), mode, "dgrad")
+    G.assert_close(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *a, L["k_vol"]), mode, "wgrad")
+    # the sequential entry point and the omitted-centre form go the same way
+    out_seq = G.run_fwd(capi, D, fused=False, plan=plan)
+    G.assert_close(out_seq, out.astype(np.float32), mode, "seq fwd")
+    plan.close()
