@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libfgms_hip.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
 HIP_SOURCES = ["fgms_api.hip", "fgms_generic.hip", "fgms_plan.hip", "fgms_mfma.hip", "fgms_small.hip", "fgms_wgrad.hip",
-               "fgms_probe.hip", "fgms_kmap.hip", "fgms_halo.hip"]
+               "fgms_probe.hip", "fgms_kmap.hip", "fgms_halo.hip", "fgms_wide.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXX = os.environ.get("CXX", "g++")

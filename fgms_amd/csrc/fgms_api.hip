@@ -292,7 +292,7 @@ bool sparse_rows(const GmsArgs &a, const Plan *plan) {
   return slots_per_pair > (need > 1.4 ? need : 1.4);
 }
 
-enum class Route { kSkinny, kHalo, kRows, kPairView, kPairs, kGeneric };
+enum class Route { kSkinny, kHalo, kRows, kPairView, kWide, kPairs, kGeneric };
 
 // Which kernel a forward / input-gradient pass takes.
 Route route_of(const GmsArgs &a, const Plan *plan) {
@@ -304,6 +304,7 @@ Route route_of(const GmsArgs &a, const Plan *plan) {
   // the kernel that keeps a tile's neighbourhood rows in LDS: on request only (it measures
   // slower than the output-stationary kernel that gathers per pair, see fgms_halo.hip)
   if (!dense && g_policy == 6 && halo_gms_supported(a, plan)) return Route::kHalo;
+  if (g_policy == 7 && wide_gms_supported(a)) return Route::kWide;
   if (!dense && g_policy != 2 && planned_gms_supported(a, plan) &&
       !(g_policy != 4 && sparse_rows(a, plan) && mfma_gms_supported(a)))
     return Route::kRows;
@@ -314,6 +315,7 @@ Route route_of(const GmsArgs &a, const Plan *plan) {
   // channels over 35 k voxels, a tie from 128 channels on (96.6 against 96.3 us at 256).
   if (g_policy == 0 && pair_view && (a.dtype == FGMS_F32 || (a.transpose_w ? a.c_out : a.c_in) <= 64))
     return Route::kPairView;
+  if (g_policy == 0 && wide_gms_supported(a)) return Route::kWide;
   return mfma_gms_supported(a) ? Route::kPairs : Route::kGeneric;
 }
 
@@ -347,6 +349,7 @@ int run_gms_one(GmsArgs a, const Plan *plan) {
     case Route::kHalo: return launch_halo_gms(a, plan);
     case Route::kRows: return launch_planned_gms(a, plan);
     case Route::kPairView: return launch_pair_view_gms(a, plan);
+    case Route::kWide: return launch_wide_gms(a);
     case Route::kPairs: return launch_mfma_gms(a);
     default: return launch_generic_gms(a);
   }

@@ -218,6 +218,10 @@ int allow_dynamic_lds(const void *kernel, size_t bytes);
 int kernel_policy();   // fgms_set_kernel_policy's value
 int num_cus();         // compute units of the current device
 int launch_mfma_gms(const GmsArgs &a);
+// Pair-stationary kernel for wide fp16 layers: 256 destination channels per workgroup, every
+// source row gathered once (fgms_wide.hip).
+bool wide_gms_supported(const GmsArgs &a);
+int launch_wide_gms(const GmsArgs &a);
 bool mfma_wgrad_supported(const WgradArgs &a);
 int launch_mfma_wgrad(const WgradArgs &a);
 // The MFMA / skinny weight gradient with its fp32 accumulator in a static device array: no

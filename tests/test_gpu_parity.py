@@ -90,6 +90,17 @@ def test_submanifold_wide_wave_tiles(capi, oracle, shape, dtype):
     check_all(capi, oracle, layer(14, shape[0], shape[1], dtype), policy=3, use_plan=True)
 
 
+@pytest.mark.parametrize("use_plan", [True, False], ids=["plan", "noplan"])
+@pytest.mark.parametrize("kind,shape", [("subm", (256, 256)), ("subm", (128, 256)), ("subm", (256, 512)),
+                                        ("subm", (512, 256)), ("down", (128, 256)), ("up", (256, 128))])
+def test_wide_pair_stationary_kernel(capi, oracle, kind, shape, use_plan):
+    """The pair-stationary kernel with 256-column workgroups (fp16, a multiple of 256
+    destination channels in the pass at hand), forced where the automatic dispatch would take a
+    plan-driven kernel: forward of the (c, 256 n) layers, input gradient of the (256 n, c) ones,
+    whole and partial 256-pair tiles, several tiles per workgroup."""
+    check_all(capi, oracle, layer(31, shape[0], shape[1], np.float16, kind), policy=7, use_plan=use_plan)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
 @pytest.mark.parametrize("parts", [1, 2, 4])
 @pytest.mark.parametrize("shape", [(4, 32), (16, 16), (64, 8)], ids=lambda s: "%dx%d" % s)
@@ -141,6 +152,23 @@ def test_separate_mid(capi, oracle, fused, dtype):
         # the fused form overwrites (GEMM beta = 0, backend/spconv.cu:56): junk in out must vanish
         junk = torch.full((len(vox), 64), 7.0, dtype=D["in_feats"].dtype, device="cuda")
         G.assert_close(G.run_fwd(capi, D, fused=True, separate_mid=True, out_init=junk), ref, mode)
+
+
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "seq"])
+def test_separate_mid_wide_layer(capi, oracle, fused):
+    """The same with 256 output channels in fp16: the centre product and the scattered map both
+    run the pair-stationary kernel with 256-column workgroups."""
+    rng = np.random.default_rng(18)
+    vox = cloud(18)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vox, vox, clouds.offsets_cube(3), skip_offset=13)
+    L = clouds.make_layer(rng, imap, omap, knnz, kpos, len(vox), len(vox), 128, 256, np.float16)
+    D = G.to_dev(L)
+    ref = oracle.np_fwd(L["in_feats"], L["kernel"], knnz, imap, omap, len(vox), precompute=True)
+    capi.set_kernel_policy(0)
+    G.assert_close(G.run_fwd(capi, D, fused=fused, separate_mid=True, plan=None), ref, "fp16")
+    if fused:
+        junk = torch.full((len(vox), 256), 7.0, dtype=D["in_feats"].dtype, device="cuda")
+        G.assert_close(G.run_fwd(capi, D, fused=True, separate_mid=True, out_init=junk), ref, "fp16")
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
@@ -313,8 +341,9 @@ def test_scattered_wide_layer_takes_the_pair_stationary_kernel(capi, oracle, dty
     names = [n for n, _ in capi.profile_records()]
     capi.profile_reset()
     plan.close()
-    # (fp32: the output-stationary kernel's body over the plan's pair view, also with atomics)
-    want = "gms_pairs_kernel(fwd)" if dtype == "wide" else "gms_rows_kernel(fwd, pair view)"
+    # (fp16: the pair-stationary kernel with 256-column workgroups; fp32: the output-stationary
+    # kernel's body over the plan's pair view; both with atomics)
+    want = "gms_wide_kernel(fwd)" if dtype == "wide" else "gms_rows_kernel(fwd, pair view)"
     assert want in names and "gms_rows_kernel(fwd)" not in names, names
     ref = oracle.np_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
     G.assert_close(out, ref, G.mode_of(L["in_feats"].dtype, False), "fwd")
