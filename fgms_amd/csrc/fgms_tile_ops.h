@@ -15,13 +15,19 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_wave_barrier();
 }
 
-// Slot of 16-byte chunk c of row `row` inside a wave's staging tile
-// (rows of 2*S chunks).  8 consecutive slots cover all LDS banks once; the XOR
-// spreads the 8 rows that one b128 read pass touches over distinct slots.
+// Slot of 16-byte chunk c of row `row` inside a wave's staging tile (rows of 2*S chunks).
+// The LDS serves 16 lanes of a b128 access per clock, 256 bytes across all banks: 16 slots.
+// A fragment read has 16 consecutive rows ask for the same chunk; with 128-byte rows (S = 4)
+// two rows share a 256-byte span, so the XOR goes by row / 2: rows r and r + 1 sit in the two
+// halves of a span, and the eight row pairs of a pass land on eight different slots of their
+// half.  (XOR by row % 8 had rows r and r + 8 collide: measured 137 against 255 bytes per
+// clock and CU for this read.)  The writes of a staged gather (8 lanes per row, 2 rows per
+// pass) are conflict-free either way.
 template <int S>
 __device__ __forceinline__ int a_slot(int row, int c) {
   constexpr int C = 2 * S;
-  return row * C + (c ^ ((row / (8 / C)) % C));
+  if constexpr (C == 8) return row * C + (c ^ ((row >> 1) & 7));
+  else return row * C + (c ^ ((row / (8 / C)) % C));
 }
 
 // --- forward weights straight from the caller's tensor (fp16) -----------------------
