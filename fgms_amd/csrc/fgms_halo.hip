@@ -20,10 +20,17 @@
 // accumulators persist, lanes whose neighbour is not resident read a row of zeros).
 //
 // Measured on MI355X, 64 -> 64 fp16 over 200 k voxels (2.1 M pairs): 57 us per pass against
-// 50 us for the kernel that gathers per pair (gms_rows_kernel), although it moves a third of
-// the bytes through L1: with 128 accumulator registers a CU holds 8 waves, and a tile's 14 us
+// 50 us for the kernel that gathers per pair (gms_rows_kernel).  It brings a sixth of the row
+// bytes into the CU (42 MB of neighbourhood rows against 270 MB of gathers) and reads half as
+// much from HBM (FETCH_SIZE 64 MB against 138 MB, L2 hit rate 85 % against 69 %), but with tiles
+// of 128 rows an offset's 8 KB of weights serve only 128 rows, 225 MB of weight reads per
+// pass against 84 MB, so the L1 asks the L2 for about as much as before (TCP_TCC_READ_REQ
+// 2.8 M against 3.1 M), and with 128 accumulator registers a CU holds 8 waves: a tile's 14 us
 // are mostly memory round trips those few waves cannot cover (neighbourhood load 2.9 us, the
 // offsets' weight fetches 8 us for 1.9 us of MFMA work, reduction and row update 3.5 us).
+// Tiles of 256 rows halve the weight reads but need 256 accumulator registers per wave or
+// rows split over more waves, which was measured too (64 - 66 us: waves own rows, an offset's
+// weights pass through LDS behind a workgroup barrier per offset).
 // A weight-stationary variant (one persistent workgroup per CU, every wave keeping the B
 // fragments of its three or four offsets in registers for the whole launch, per-tile sums
 // combined in LDS) was measured too: ds_add_f32 runs at about a lane per clock, 620 us per pass;
