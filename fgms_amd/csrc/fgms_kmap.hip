@@ -13,15 +13,13 @@
 //               keeps the smallest row index (atomicMin)
 //   2. lookup   one thread per (offset, output row): probe, write the hit (or
 //               -1) into a [k_vol][n_out] table, count hits per 256-row block
-//   3. scan     exclusive prefix sum over the (offset, block) counts (rocPRIM)
+//   3. scan     exclusive prefix sum over the (offset, block) counts (one workgroup)
 //   4. write    hits are compacted in (offset, row) order: block base from the
 //               scan, rank inside the block from wave ballots
 #include <stdlib.h>
 #include <string.h>
 
 #include <vector>
-
-#include <rocprim/device/device_scan.hpp>
 
 #include "fgms_device.h"
 #include "fgms_internal.h"
@@ -33,6 +31,47 @@ constexpr unsigned long long kEmptyKey = ~0ull;
 constexpr int kCoordBits = 21;
 constexpr long long kCoordBias = 1ll << (kCoordBits - 1);   // coordinates in [-2^20, 2^20)
 constexpr int kBlock = 256;
+
+// Exclusive prefix sum of n ints by one workgroup of 1024 threads, 4096 values a round: every
+// thread takes four neighbouring values (the loads of a wave are contiguous), the waves scan
+// their threads' sums with lane shuffles, the 16 wave totals go through LDS, and the sum of the
+// rounds so far is carried in a register.  The counts are few (offsets x 256-row blocks: 21 k
+// for 200 k voxels), so one workgroup is enough.
+__global__ __launch_bounds__(1024) void kmap_scan_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out,
+                                                         size_t n) {
+  __shared__ int wave_totals[2][16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int carry = 0, round = 0;
+  for (size_t base = 0; base < n; base += 4096, round ^= 1) {
+    const size_t i = base + (size_t)tid * 4;
+    int v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = i + j < n ? in[i + j] : 0;
+    const int mine = v[0] + v[1] + v[2] + v[3];
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) wave_totals[round][wave] = incl;
+    __syncthreads();      // the other buffer is written next round, after every wave has passed this barrier
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int t = wave_totals[round][w];
+      before += w < wave ? t : 0;
+      total += t;
+    }
+    int run = carry + before + incl - mine;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (i + j < n) out[i + j] = run;
+      run += v[j];
+    }
+    carry += total;
+  }
+}
 
 __device__ __forceinline__ bool pack_key(long long x, long long y, long long z, unsigned long long &key) {
   x += kCoordBias; y += kCoordBias; z += kCoordBias;
@@ -214,12 +253,8 @@ int build_kernel_map_impl(const int32_t *in_coords, int64_t n_in, const int32_t 
   auto *bases = (int32_t *)alloc(n_counts * sizeof(int32_t));
   auto *offs = (int32_t *)alloc((size_t)k_vol * 3 * sizeof(int32_t));
   auto *flags = (int32_t *)alloc(4 * sizeof(int32_t));      // [0] bad coordinate, [1] total
-  size_t scan_bytes = 0;
-  bool ok = keys && vals && table && counts && bases && offs && flags &&
-            rocprim::exclusive_scan(nullptr, scan_bytes, counts, bases, 0, n_counts,
-                                    rocprim::plus<int32_t>(), s) == hipSuccess;
-  void *scan_tmp = ok ? alloc(scan_bytes) : nullptr;
-  if (!ok || !scan_tmp) {
+  const bool ok = keys && vals && table && counts && bases && offs && flags;
+  if (!ok) {
     release();
     set_error("fgms_build_kernel_map: temporary allocation failed");
     return FGMS_E_NOMEM;
@@ -260,8 +295,7 @@ int build_kernel_map_impl(const int32_t *in_coords, int64_t n_in, const int32_t 
                                                                                             k_vol / 2 + 1, counts);
     }
   }
-  if (rocprim::exclusive_scan(scan_tmp, scan_bytes, counts, bases, 0, n_counts, rocprim::plus<int32_t>(), s) != hipSuccess)
-    return fail("prefix sum failed");
+  kmap_scan_kernel<<<1, 1024, 0, s>>>(counts, bases, n_counts);
   if (n_out > 0) {
     ProfileScope prof("kmap_write_kernel", s);
     kmap_write_kernel<<<dim3((unsigned)n_blocks, (unsigned)k_vol), kBlock, 0, s>>>(
