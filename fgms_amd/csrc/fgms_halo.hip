@@ -31,12 +31,25 @@
 // Tiles of 256 rows halve the weight reads but need 256 accumulator registers per wave or
 // rows split over more waves, which was measured too (64 - 66 us: waves own rows, an offset's
 // weights pass through LDS behind a workgroup barrier per offset).
-// A weight-stationary variant (one persistent workgroup per CU, every wave keeping the B
-// fragments of its three or four offsets in registers for the whole launch, per-tile sums
-// combined in LDS) was measured too: ds_add_f32 runs at about a lane per clock, 620 us per pass;
-// with plain stores in its place (wrong sums, timing only) still 75 us, because the compiler
-// waits for every outstanding direct-to-LDS load before any LDS access that follows it, which
-// undoes the double buffering of the neighbourhood rows.
+// Weight-stationary variants (one persistent workgroup per CU that keeps every offset's B
+// fragments in registers for the whole launch, so that a tile brings in nothing but its
+// neighbourhood rows; next tile's rows streamed into a second LDS buffer meanwhile; the waves
+// split the offsets, k mod 4, and their partial tiles meet in LDS) were measured too:
+//   * 8 waves (offset group x column half, 112 fragment registers each): 60 - 78 us.  Both
+//     column halves read the same A fragments, and with 16 waves' worth of 16-byte row reads
+//     per 128 MFMA clocks the LDS is the limit, not the matrix pipe.
+//   * 4 waves with 512 registers each (224 fragment registers, held in the accumulation
+//     register file through register constraints and hand-written MFMAs, since the compiler
+//     spills MFMA B operands rather than place them there; A fragments read from inline
+//     assembly one 32-row block ahead of their products): parity-exact, 71 us.  Without the
+//     products 41 us, without the reduction and row update 55 us: a (offset, block) step takes
+//     about 600 clocks against 256 of MFMA issue with a single wave per SIMD to cover LDS
+//     latency, the four partial tiles cost 128 four-byte LDS writes per wave and three barriers
+//     per tile (2.7 us), and with 6.1 tiles per workgroup and 2 x different tile lengths the
+//     static tile runs end 25 % apart.
+//   * the first attempt combined the partial tiles with ds_add_f32 (about a lane per clock):
+//     620 us.
+// 27 offsets x 64 x 64 weights fill the registers of a CU; nothing is left to hide latency with.
 // So this path is opt-in: the tables are built by fgms_plan_create_coords only, and the
 // kernel runs under kernel policy 6 only.
 #include <stdlib.h>
@@ -59,6 +72,13 @@ constexpr int kHaloThreads = 256; // the kernel's workgroup
 constexpr int kBuildThreads = kHaloTile;   // the plan kernel's: one thread per position of a tile
 constexpr int kHashSlots = 8192;  // >= 64 offsets x 128 rows; 27 x 256 = 6 912 keys fit too
 constexpr unsigned short kNoNbr = 0xFFFF;
+
+// Where the neighbour-list position of (tile, offset k, position t of the tile) sits in the
+// table: the four 32-row blocks' entries of one row-of-block next to each other, so that an
+// MFMA lane (row t % 32 of every block) fetches its four entries of an offset in one 8-byte load.
+__host__ __device__ __forceinline__ size_t lnbr_slot(int tile, int k_vol, int k, int t) {
+  return (((size_t)tile * k_vol + k) * 32 + t % 32) * 4 + t / 32;
+}
 
 // ---------------------------------------------------------------------------------------
 // Row orders.
@@ -99,7 +119,7 @@ __global__ void invert_order_kernel(const int32_t *__restrict__ order, int n, in
 //   inv_src   [n_src]         source row -> source position (nullptr: identity)
 //   order_src [n_src]         source position -> source row (nullptr: identity)
 // out: order_pad [n_tiles * kHaloTile], rows [n_tiles][list_cap], count [n_tiles],
-//      lnbr [k_vol][n_tiles * kHaloTile], mask32 [n_tiles * kHaloTile / 32];
+//      lnbr [n_tiles][k_vol][32][4] (see lnbr_slot), mask32 [n_tiles * kHaloTile / 32];
 //      flags[0] = 1 if some list did not fit, flags[1] += rounds beyond the first.
 __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
     const int32_t *__restrict__ nbr, const int32_t *__restrict__ plan_pos, const int32_t *__restrict__ order_dst,
@@ -182,7 +202,7 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
       flags[0] = 1;
       count[tile] = 0;
     }
-    for (int k = 0; k < k_vol; ++k) lnbr[(size_t)k * n_pad + p] = kNoNbr;
+    for (int k = 0; k < k_vol; ++k) lnbr[lnbr_slot(tile, k_vol, k, tid)] = kNoNbr;
     if (tid % 32 == 0) mask32[p / 32] = 0;
     return;
   }
@@ -204,8 +224,11 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
       }
       __syncthreads();
     }
-  for (int i = tid; i < u; i += kBuildThreads)
-    rows[(size_t)tile * list_cap + i] = order_src ? order_src[list[i]] : list[i];
+  // (padded to a multiple of 8 with the last row: the kernels fetch row numbers in groups of 8)
+  for (int i = tid; i < min((u + 7) / 8 * 8, list_cap); i += kBuildThreads) {
+    const int key = list[min(i, u - 1)];
+    rows[(size_t)tile * list_cap + i] = order_src ? order_src[key] : key;
+  }
   if (tid == 0) {
     count[tile] = u;
     const int extra = (u + kHaloCap - 1) / kHaloCap - 1;
@@ -225,7 +248,7 @@ __global__ __launch_bounds__(kBuildThreads) void halo_build_kernel(
       }
       lid = (unsigned short)lo;
     }
-    lnbr[(size_t)k * n_pad + p] = lid;
+    lnbr[lnbr_slot(tile, k_vol, k, tid)] = lid;
     const unsigned long long b = __ballot(g >= 0);
     const unsigned half = (tid & 32) ? (unsigned)(b >> 32) : (unsigned)b;
     if (half) mine |= 1ull << k;
@@ -276,7 +299,6 @@ __global__ __launch_bounds__(kHaloThreads, 2) void gms_halo_kernel(
   const int per_xcd = (n_tiles + 7) / 8;
   const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if ((int)(blockIdx.x / 8) >= per_xcd || tile >= n_tiles) return;
-  const int n_pad = n_tiles * kHaloTile;
   const int p0 = tile * kHaloTile;
   const int cd0 = blockIdx.y * 64;
   const int count = hcount[tile];
@@ -345,11 +367,11 @@ __global__ __launch_bounds__(kHaloThreads, 2) void gms_halo_kernel(
       }
     wave_lds_fence();
   };
-  const int my_pos = p0 + r;
   auto idx_issue = [&](int (&ix)[kBlocks], int k) {
-    const unsigned short *lk = lnbr + (size_t)k * n_pad + my_pos;
+    typedef unsigned short ushort4v __attribute__((ext_vector_type(4)));
+    const ushort4v e = *reinterpret_cast<const ushort4v *>(lnbr + lnbr_slot(tile, k_vol, k, r));
 #pragma unroll
-    for (int b = 0; b < kBlocks; ++b) ix[b] = lk[b * 32];
+    for (int b = 0; b < kBlocks; ++b) ix[b] = e[b];
   };
   auto grab = [&]() {
     int i = 0;

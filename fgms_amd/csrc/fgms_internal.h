@@ -97,13 +97,13 @@ struct WgradArgs {
 };
 
 // One direction of a plan's tile tables for the kernels that keep a tile's neighbourhood in
-// LDS (fgms_halo.hip): destination rows in a spatially compact order, cut into tiles of 256.
+// LDS (fgms_halo.hip): destination rows in a spatially compact order, cut into tiles of 128.
 struct HaloSide {
-  int32_t *order;               // [n_tiles * 256] position -> destination row, -1 = padding
-  int32_t *rows;                // [n_tiles][list_cap] the tile's distinct source rows, in source order
+  int32_t *order;               // [n_tiles * 128] position -> destination row, -1 = padding
+  int32_t *rows;                // [n_tiles][list_cap] the tile's distinct source rows, in source order (padded to 8s)
   int32_t *count;               // [n_tiles] how many
-  unsigned short *lnbr;         // [k_vol][n_tiles * 256] index into the tile's list, 0xFFFF = no neighbour
-  unsigned long long *mask32;   // [n_tiles * 8] offsets in use per block of 32 positions
+  unsigned short *lnbr;         // [n_tiles][k_vol][32][4] index into the tile's list by (row of block, block), 0xFFFF = no neighbour
+  unsigned long long *mask32;   // [n_tiles * 4] offsets in use per block of 32 positions
   int n_tiles, list_cap;
   int64_t extra_rounds;         // sum over tiles of the LDS rounds beyond the first
   bool ok;                      // built and every tile's list fitted list_cap
