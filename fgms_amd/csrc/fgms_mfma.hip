@@ -80,8 +80,8 @@ __device__ __forceinline__ void load_weights_bf3(int4v *__restrict__ w_lds,
 }
 
 // acc[mt][nt] += A(slab) x W(slab).
-template <typename T, int NT, int S>
-__device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+template <typename T, int NT, int S, int MT>
+__device__ __forceinline__ void mma_slab(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                          const int4v *__restrict__ w_lds, int slab, int lane) {
   const int h = lane / 32, r = lane % 32;
 #pragma unroll
@@ -90,7 +90,7 @@ __device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[((slab * S + s) * NT + nt) * 64 + lane];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
@@ -99,8 +99,8 @@ __device__ __forceinline__ void mma_slab(float16v (&acc)[2][NT], const int4v *__
 }
 
 // acc[mt][nt] += A(slab) x W(slab), weights as raw_weight_frag reads them.
-template <typename T, int NT, int S>
-__device__ __forceinline__ void mma_slab_raw(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+template <typename T, int NT, int S, int MT>
+__device__ __forceinline__ void mma_slab_raw(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                              const int4v *__restrict__ w_lds, int lane) {
   const int h = lane / 32, r = lane % 32;
 #pragma unroll
@@ -109,7 +109,7 @@ __device__ __forceinline__ void mma_slab_raw(float16v (&acc)[2][NT], const int4v
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) b[nt] = raw_weight_frag<NT, S>(w_lds, s, nt, lane);
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
@@ -123,8 +123,8 @@ __device__ __forceinline__ void mma_slab_raw(float16v (&acc)[2][NT], const int4v
 // MFMA lane wants are one 16-byte piece of row ci.  A stage's weight tile (NT*32 rows ci x
 // 2*S chunks of the co slab) goes to LDS as it lies in memory, swizzled like a wave's
 // staging tile of gathered rows, and a fragment is one 16-byte read.  No re-layout at all.
-template <typename T, int NT, int S>
-__device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+template <typename T, int NT, int S, int MT>
+__device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                               const int4v *__restrict__ w_lds, int lane) {
   const int h = lane / 32, r = lane % 32;
 #pragma unroll
@@ -133,7 +133,7 @@ __device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[2][NT], const int4
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[a_slot<S>(nt * 32 + r, h * S + s)];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
@@ -179,10 +179,11 @@ __device__ __forceinline__ void split_and_store(int4v *__restrict__ tile, const 
 }
 
 // registers -> LDS for the split tile of gathered rows (absent rows as zeros).
-__device__ __forceinline__ void gather_commit_bf3(int4v *__restrict__ a_lds, int4v (&v)[8],
-                                                  const int (&g)[8], int lane) {
+template <int N>
+__device__ __forceinline__ void gather_commit_bf3(int4v *__restrict__ a_lds, int4v (&v)[N],
+                                                  const int (&g)[N], int lane) {
 #pragma unroll
-  for (int it = 0; it < 8; ++it) {
+  for (int it = 0; it < N; ++it) {
     const int slot = it * 64 + lane;
     const float4v x = g[it] < 0 ? float4v{0.f, 0.f, 0.f, 0.f} : __builtin_bit_cast(float4v, v[it]);
     split_and_store(a_lds, x, slot / 8, slot % 8, lane);
@@ -190,8 +191,8 @@ __device__ __forceinline__ void gather_commit_bf3(int4v *__restrict__ a_lds, int
 }
 
 // acc[mt][nt] += A(slab) x W(slab), both split; weights in LDS as [k-step][nt][hi, lo][lane].
-template <int NT>
-__device__ __forceinline__ void mma_slab_bf3(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+template <int NT, int MT>
+__device__ __forceinline__ void mma_slab_bf3(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                              const int4v *__restrict__ w_lds, int lane) {
   const int h = lane / 32, r = lane % 32;
 #pragma unroll
@@ -203,7 +204,7 @@ __device__ __forceinline__ void mma_slab_bf3(float16v (&acc)[2][NT], const int4v
       bl[nt] = __builtin_bit_cast(bf16x8, w_lds[((s * NT + nt) * 2 + 1) * 64 + lane]);
     }
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const bf16x8 ah = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 0, s * 2 + h)]);
       const bf16x8 al = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 1, s * 2 + h)]);
 #pragma unroll
@@ -218,8 +219,8 @@ __device__ __forceinline__ void mma_slab_bf3(float16v (&acc)[2][NT], const int4v
 
 // The same for the input gradient: the weight tile (NT*32 rows of W[k], the slab's 32 columns)
 // was split on its way to LDS like a tile of gathered rows (RAW = 4).
-template <int NT>
-__device__ __forceinline__ void mma_slab_bf3t(float16v (&acc)[2][NT], const int4v *__restrict__ a_lds,
+template <int NT, int MT>
+__device__ __forceinline__ void mma_slab_bf3t(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                               const int4v *__restrict__ w_lds, int lane) {
   const int h = lane / 32, r = lane % 32;
 #pragma unroll
@@ -231,7 +232,7 @@ __device__ __forceinline__ void mma_slab_bf3t(float16v (&acc)[2][NT], const int4
       bl[nt] = __builtin_bit_cast(bf16x8, w_lds[a_bf_slot(nt * 32 + r, 1, s * 2 + h)]);
     }
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const bf16x8 ah = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 0, s * 2 + h)]);
       const bf16x8 al = __builtin_bit_cast(bf16x8, a_lds[a_bf_slot(mt * 32 + r, 1, s * 2 + h)]);
 #pragma unroll
@@ -280,29 +281,30 @@ __global__ void pack_weights_bf3_kernel(const float *__restrict__ w, int4v *__re
 // Row gathers in two steps, so that the loads of one slab run under the MFMAs of the
 // previous one: issue (global -> registers, absent rows read row 0) and commit
 // (registers -> the wave's LDS tile, absent rows as zeros; waits for the loads).
-template <typename T, int S>
-__device__ __forceinline__ void gather_issue(int4v (&v)[2 * S], int (&g)[2 * S],
+// (N chunks per lane: 2 * S for a wave tile of 64 rows, S for one of 32)
+template <typename T, int S, int N>
+__device__ __forceinline__ void gather_issue(int4v (&v)[N], int (&g)[N],
                                              const int *__restrict__ idx,
                                              const T *__restrict__ src, int c_src, int slab,
                                              int lane) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
 #pragma unroll
-  for (int it = 0; it < C; ++it) g[it] = idx[(it * 64 + lane) / C];
+  for (int it = 0; it < N; ++it) g[it] = idx[(it * 64 + lane) / C];
 #pragma unroll
-  for (int it = 0; it < C; ++it) {
+  for (int it = 0; it < N; ++it) {
     const int c = (it * 64 + lane) % C;
     v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(g[it], 0) * c_src +
                                              (size_t)(slab * C + c) * E);
   }
 }
 
-template <int S>
-__device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (&v)[2 * S],
-                                              const int (&g)[2 * S], int lane) {
+template <int S, int N>
+__device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (&v)[N],
+                                              const int (&g)[N], int lane) {
   constexpr int C = 2 * S;
 #pragma unroll
-  for (int it = 0; it < C; ++it) {
+  for (int it = 0; it < N; ++it) {
     const int slot = it * 64 + lane;
     a_lds[a_slot<S>(slot / C, slot % C)] = g[it] < 0 ? int4v{0, 0, 0, 0} : v[it];
   }
@@ -404,7 +406,10 @@ __global__ __launch_bounds__(kThreads) void gms_pairs_kernel(
 // the input gradient in split bf16, weights read as they lie and split on their way to LDS;
 // RAW = 0: the re-laid copy pack_weight_elements makes.
 // (block_x, block_y, block_z) of a grid (tiles, column tiles, grid_z parts of a tile).
-template <typename T, int NT, int S, int RAW>
+// MT: 32-row MFMA tiles per wave.  2 (a workgroup tile of 256 rows) is the layout every plan
+// table is made for; 1 (tiles of 128 rows, half the work per wave and stage) serves launches
+// too small to fill the chip, where a tile's chain of stages is all there is to the duration.
+template <typename T, int NT, int S, int RAW, int MT = 2>
 __device__ __forceinline__ void gms_rows_body(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
@@ -427,10 +432,12 @@ __device__ __forceinline__ void gms_rows_body(
   const int nts = c_dst / 32;
   int4v *w_lds = lds;                                     // [2][WCH]
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  int4v *a_lds = lds + 2 * WCH + wave * (kWaveRows * C);
-  int *idx_all = reinterpret_cast<int *>(lds + 2 * WCH + kWaves * (kWaveRows * C));
-  int *gidx = idx_all + wave * 2 * kWaveRows;
-  int *didx = gidx + kWaveRows;
+  constexpr int WR = MT * 32;                             // rows per wave
+  constexpr int TR = kWaves * WR;                         // rows per workgroup tile
+  int4v *a_lds = lds + 2 * WCH + wave * (WR * C);
+  int *idx_all = reinterpret_cast<int *>(lds + 2 * WCH + kWaves * (WR * C));
+  int *gidx = idx_all + wave * 2 * WR;
+  int *didx = gidx + WR;
   const int nt0 = block_y * NT;
   const int4v *packed4 = reinterpret_cast<const int4v *>(packed);
   const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
@@ -443,15 +450,16 @@ __device__ __forceinline__ void gms_rows_body(
     tile = entry & 0xFFFFFF;
     if (grid_z == 1) k_first = entry >> 24;
   }
-  const int row0 = tile * kTileRows + wave * kWaveRows;
+  const int row0 = tile * TR + wave * WR;
   const int my_row = row0 + lane;
-  const bool in_range = my_row < n_dst;
+  const bool owns_row = MT == 2 || lane < WR;             // (lanes past a 32-row wave tile own no row)
+  const bool in_range = owns_row && my_row < n_dst;
   // that offset's neighbour index, fetched while the masks are still on their way: at the
   // start of a launch every workgroup walks this chain of dependent loads at the same time
   // and nothing else covers it (0.4 us of a 46 us launch)
   int g_first = -1;
   if (k_first >= 0 && in_range) g_first = nbr[(size_t)k_first * nbr_stride + my_row];
-  didx[lane] = in_range ? (perm ? perm[my_row] : my_row) : -1;   // my_row is a position in the plan's row order
+  if (owns_row) didx[lane] = in_range ? (perm ? perm[my_row] : my_row) : -1;   // my_row is a position in the plan's row order
 
   // which offsets touch this wave's rows / this workgroup's rows (from the plan)
   const unsigned long long wave_mask = row0 < n_dst ? block_masks[row0 / 64] : 0ull;
@@ -491,9 +499,9 @@ __device__ __forceinline__ void gms_rows_body(
     }
   }
 
-  float16v acc[2][NT];
+  float16v acc[MT][NT];
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -554,11 +562,12 @@ __device__ __forceinline__ void gms_rows_body(
   if (todo) todo &= todo - 1;
   bool active = (wave_mask >> k) & 1;
   int4v wreg[NW];
-  int4v v[C];
-  int gsel[C];
+  constexpr int NV = MT * S;                              // row chunks per lane and stage
+  int4v v[NV];
+  int gsel[NV];
 
   // prologue: stage 0 goes straight to LDS
-  gidx[lane] = k_first >= 0 ? g_first : (in_range ? nbr[(size_t)k * nbr_stride + my_row] : -1);
+  if (owns_row) gidx[lane] = k_first >= 0 ? g_first : (in_range ? nbr[(size_t)k * nbr_stride + my_row] : -1);
   int g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * nbr_stride + my_row] : -1;
   wave_lds_fence();
   weights_issue(wreg, k, 0);
@@ -575,7 +584,7 @@ __device__ __forceinline__ void gms_rows_body(
     const bool next_active = has_next && ((wave_mask >> nk) & 1);
     if (has_next) {
       if (nk != k) {          // the row loads that used the old indices were issued a stage ago
-        gidx[lane] = g_nxt;
+        if (owns_row) gidx[lane] = g_nxt;
         wave_lds_fence();
       }
     }
@@ -599,11 +608,11 @@ __device__ __forceinline__ void gms_rows_body(
           else b[nt] = wl[(s * NT + nt) * 64 + lane];
         }
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
+        for (int mt = 0; mt < MT; ++mt) {
           const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
-          const int it = s * 2 + mt;                       // one of the C = 2 * S row loads
+          const int it = s * MT + mt;                      // one of the MT * S row loads
           gsel[it] = gidx[(it * 64 + lane) / C];
           v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(gsel[it], 0) * c_src +
                                                    (size_t)(nslab * C + (it * 64 + lane) % C) * E);
@@ -647,8 +656,8 @@ __device__ __forceinline__ void gms_rows_body(
   }
 }
 
-template <typename T, int NT, int S, int RAW>
-__global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
+template <typename T, int NT, int S, int RAW, int MT = 2>
+__global__ __launch_bounds__(kThreads, MT == 1 ? 4 : (NT == 4 ? 2 : 3)) void gms_rows_kernel(
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
@@ -662,8 +671,8 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void gms_rows_kernel(
     }
     block_x -= side.blocks;
   }
-  gms_rows_body<T, NT, S, RAW>(src, packed, dst, nbr, block_masks, perm, tile_order, n_dst, k_vol, c_src,
-                               c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z, pair_view);
+  gms_rows_body<T, NT, S, RAW, MT>(src, packed, dst, nbr, block_masks, perm, tile_order, n_dst, k_vol, c_src,
+                                   c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z, pair_view);
 }
 
 // ---------------------------------------------------------------------------
@@ -759,6 +768,50 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   return FGMS_OK;
 }
 
+// FGMS_HALF_TILES=0 keeps small launches on 256-row tiles (for comparison).
+bool half_tiles_enabled() {
+  static const bool on = !(getenv("FGMS_HALF_TILES") && atoi(getenv("FGMS_HALF_TILES")) == 0);
+  return on;
+}
+
+// Grid of an output-stationary launch over n_dst destination rows: tiles of 256 rows from the
+// plan's tile table where there is one (`table_grid` entries), else plain tiles of 256 or --
+// where those still fit the chip's workgroup slots in one round -- of 128 rows (32 per wave:
+// twice the waves, half the work per wave and stage; such a launch lasts as long as one
+// tile's chain of stages).  A launch that then fills less than half of the slots shares every
+// tile between two workgroups, each taking half of the tile's stages and adding its part with
+// atomics: twice the workgroups, half the critical path.  (Two parts only: the sum of two
+// partial results does not depend on their order.  On launches that fill the chip the atomics
+// cost more than the split gains.)  The standalone and the one-grid backward launch share this
+// choice, so that their input gradients agree bit for bit; an input gradient takes the small
+// tiles only for long chains (24 stages and more), since in the backward launch its
+// workgroups share the chip with the weight gradient's and twice as many of them delay those.
+// Measured (MI355X, step = fwd + dgrad + wgrad): 32 -> 32 fp32 over 20 k voxels 64.0 -> 56.6 us,
+// 64 -> 128 fp16 stride-2 (49 k output rows) forward 21.5 -> 19.7 us; the 8-offset input
+// gradient of the transposed layer inside the backward launch 34.6 -> 35.9 us, hence the rule.
+struct RowsGrid {
+  bool half_tiles;
+  unsigned gx, gz;
+  int part_stages;
+};
+RowsGrid rows_grid(int64_t n_dst, unsigned gy, int stages, bool can_half, bool has_table, int table_grid,
+                   bool pair_view, int wgs_per_cu, bool input_gradient) {
+  RowsGrid g{};
+  g.half_tiles = can_half && half_tiles_enabled() && !has_table && !pair_view &&
+                 (!input_gradient || stages >= 24) &&
+                 (int64_t)((n_dst + 127) / 128) * gy <= (int64_t)num_cus() * 4;
+  const int tile_rows = g.half_tiles ? kTileRows / 2 : kTileRows;
+  g.gx = has_table ? (unsigned)table_grid : (unsigned)((n_dst + tile_rows - 1) / tile_rows);
+  const int64_t slots = (int64_t)num_cus() * (g.half_tiles ? 4 : wgs_per_cu);
+  g.gz = 1;
+  g.part_stages = 1;
+  if (!pair_view && (int64_t)g.gx * gy * 2 <= slots && stages >= 8) {
+    g.part_stages = (stages + 1) / 2;
+    g.gz = 2;
+  }
+  return g;
+}
+
 // FGMS_RAW_WEIGHTS=0 keeps the forward pass on re-laid weights (for comparison).
 bool raw_weights_enabled() {
   static const bool on = !(getenv("FGMS_RAW_WEIGHTS") && atoi(getenv("FGMS_RAW_WEIGHTS")) == 0);
@@ -801,35 +854,37 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
     int rc = pack_weights<T>(a, s, &packed);
     if (rc != FGMS_OK) return rc;
   }
-  const unsigned gx = tile_order ? (unsigned)tile_grid : (unsigned)((a.n_dst + kTileRows - 1) / kTileRows);
+  const int slabs = s.c_src / (2 * S * s.E);
+  const unsigned gy = (unsigned)(s.c_dst / (32 * NT));
+  constexpr bool kCanHalf = NT != 4;
+  const RowsGrid rg = rows_grid(a.n_dst, gy, a.k_vol * slabs, kCanHalf, tile_order != nullptr, tile_grid, pair_view,
+                                NT == 4 ? 2 : 3, a.transpose_w);
+  const bool half_tiles = rg.half_tiles;
+  const size_t lds_rows = half_tiles ? s.lds_rows_bytes - (size_t)kWaves * 32 * (2 * S * 16 + 2 * sizeof(int))
+                                     : s.lds_rows_bytes;
+  const unsigned gx = rg.gx;
   if (gx == 0) return a.side.kind ? launch_side_job(a.side, a.stream) : FGMS_OK;
   constexpr bool kCanRaw = NT != 4;
-  auto kern = raw == 4   ? gms_rows_kernel<T, NT, S, kCanSplit ? 4 : 0>
+  constexpr int kHalfMT = kCanHalf ? 1 : 2;
+  auto kern = half_tiles ? (raw == 4   ? gms_rows_kernel<T, NT, S, kCanSplit ? 4 : 0, kHalfMT>
+                            : raw == 3 ? gms_rows_kernel<T, NT, S, kCanSplit ? 3 : 0, kHalfMT>
+                            : raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0, kHalfMT>
+                            : raw == 1 ? gms_rows_kernel<T, NT, S, kCanRaw && sizeof(T) == 2 ? 1 : 0, kHalfMT>
+                                       : gms_rows_kernel<T, NT, S, 0, kHalfMT>)
+              : raw == 4 ? gms_rows_kernel<T, NT, S, kCanSplit ? 4 : 0>
               : raw == 3 ? gms_rows_kernel<T, NT, S, kCanSplit ? 3 : 0>
               : raw == 2 ? gms_rows_kernel<T, NT, S, kCanRaw ? 2 : 0>
               : raw == 1 ? gms_rows_kernel<T, NT, S, kCanRaw && sizeof(T) == 2 ? 1 : 0>
                          : gms_rows_kernel<T, NT, S, 0>;
-  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)s.lds_rows_bytes); if (rc_lds != FGMS_OK) return rc_lds; }
-  // A launch that fills less than half of the chip's workgroup slots shares every
-  // tile between two workgroups, each taking half of the tile's offsets and adding
-  // its part with atomics: twice the workgroups, half the critical path.  (Two
-  // parts only: the sum of two partial results does not depend on their order.
-  // On launches that fill the chip the atomics cost more than the split gains.)
-  const int slabs = s.c_src / (2 * S * s.E);
-  const unsigned gy = (unsigned)(s.c_dst / (32 * NT));
-  const int64_t slots = (int64_t)num_cus() * (NT == 4 ? 2 : 3);
-  int part_stages = 0;
-  unsigned gz = 1;
-  if (!pair_view && (int64_t)gx * gy * 2 <= slots && a.k_vol * slabs >= 8) {
-    part_stages = (a.k_vol * slabs + 1) / 2;
-    gz = 2;
-  }
+  { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds_rows); if (rc_lds != FGMS_OK) return rc_lds; }
+  const int part_stages = rg.gz > 1 ? rg.part_stages : 0;
+  const unsigned gz = rg.gz;
   {
     ProfileScope prof(pair_view ? (a.transpose_w ? "gms_rows_kernel(dgrad, pair view)" : "gms_rows_kernel(fwd, pair view)") :raw == 4   ? "gms_rows_kernel(dgrad, bf16x3)"
                       : raw == 3 ? "gms_rows_kernel(fwd, bf16x3)"
                       : a.transpose_w ? "gms_rows_kernel(dgrad)" : "gms_rows_kernel(fwd)",
                       a.stream);
-    kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, s.lds_rows_bytes, a.stream>>>(
+    kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, lds_rows, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
         s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side, pair_view ? 1 : 0);
   }
@@ -850,7 +905,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
 // dealing the two kinds alternately or the weight gradient first measured 1-2 us slower).
 // Their count is a multiple of 8, so that a workgroup's index mod 8, its XCD, is what the
 // plan's XCD-aware orders of either kind assume.
-template <typename T, int NT, int S, int BI, int BJ, int RAWD>
+template <typename T, int NT, int S, int BI, int BJ, int RAWD, int MT = 2>
 __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
     const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
@@ -863,8 +918,8 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
   const int rows_total = row_x * row_y * row_z;
   if ((int)blockIdx.x < rows_total) {
     const int bx = blockIdx.x % row_x, rest = blockIdx.x / row_x;
-    gms_rows_body<T, NT, S, RAWD>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
-                               part_stages, bx, rest % row_y, rest / row_y, row_z);
+    gms_rows_body<T, NT, S, RAWD, MT>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
+                                      part_stages, bx, rest % row_y, rest / row_y, row_z);
   } else {
     const int j = blockIdx.x - rows_total;
     if constexpr (BI <= 2 && BJ <= 2)
@@ -886,24 +941,25 @@ template <typename T, int NT, int S, int BI, int BJ>
 int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArgs &w, const WgradGeometry &g,
                  float *acc32) {
   // the input gradient's grid, as launch_rows lays it out (tiles padded to a multiple of 8)
-  const unsigned tiles = p->tile_in ? (unsigned)p->tile_grid_in : (unsigned)((d.n_dst + kTileRows - 1) / kTileRows);
-  const unsigned row_x = (tiles + 7) / 8 * 8;
   const int slabs = s.c_src / (2 * S * s.E);
   const unsigned row_y = (unsigned)(s.c_dst / (32 * NT));
-  const int64_t slots = (int64_t)num_cus() * (NT == 4 ? 2 : 3);
-  int part_stages = 1;
-  unsigned row_z = 1;
-  if ((int64_t)tiles * row_y * 2 <= slots && d.k_vol * slabs >= 8) {
-    part_stages = (d.k_vol * slabs + 1) / 2;
-    row_z = 2;
-  }
+  constexpr bool kCanHalf = NT != 4;
+  const RowsGrid rg = rows_grid(d.n_dst, row_y, d.k_vol * slabs, kCanHalf, p->tile_in != nullptr, p->tile_grid_in,
+                                false, NT == 4 ? 2 : 3, true);
+  const unsigned row_x = (rg.gx + 7) / 8 * 8;
+  const int part_stages = rg.part_stages;
+  const unsigned row_z = rg.gz;
   size_t lds = g.lds;
   if (lds < s.lds_rows_bytes) lds = s.lds_rows_bytes;
   // RAWD: how the input gradient reads the weights (2: as they lie; 4: also split into bf16
   // pairs, for fp32 tensors whose caller allows tf32 precision)
   constexpr bool kCanSplit = sizeof(T) == 4 && S == 4 && NT != 4;
   const bool split = kCanSplit && d.reduced && split_bf16_enabled() && g.split;
-  auto kern = split ? bwd_fused_kernel<T, NT, S, BI, BJ, kCanSplit ? 4 : 2> : bwd_fused_kernel<T, NT, S, BI, BJ, 2>;
+  constexpr int kHalfMT = kCanHalf ? 1 : 2;
+  auto kern = rg.half_tiles ? (split ? bwd_fused_kernel<T, NT, S, BI, BJ, kCanSplit ? 4 : 2, kHalfMT>
+                                     : bwd_fused_kernel<T, NT, S, BI, BJ, 2, kHalfMT>)
+              : split       ? bwd_fused_kernel<T, NT, S, BI, BJ, kCanSplit ? 4 : 2>
+                            : bwd_fused_kernel<T, NT, S, BI, BJ, 2>;
   { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)lds); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof(split ? "bwd_fused_kernel(bf16x3)" : "bwd_fused_kernel", d.stream);

@@ -66,13 +66,13 @@ __device__ __forceinline__ int4v raw_weight_frag(const int4v *__restrict__ w_lds
 // (r / 4) * 8 + (l / 32) * 4 + r % 4 and column l % 32 of its 32x32 tile.  For
 // fp16 two lanes swap one value each so that every lane owns two neighbouring
 // columns of one row and can issue a packed 4-byte update.
-template <typename T, int NT, bool ATOMIC>
-__device__ __forceinline__ void write_tile(const float16v (&acc)[2][NT], T *__restrict__ dst,
+template <typename T, int NT, bool ATOMIC, int MT>
+__device__ __forceinline__ void write_tile(const float16v (&acc)[MT][NT], T *__restrict__ dst,
                                            const int *__restrict__ rows, int c_dst, int cd0,
                                            int lane) {
   const int h = lane / 32, col = lane % 32;
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
+  for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       if constexpr (sizeof(T) == 4) {
@@ -110,17 +110,17 @@ __device__ __forceinline__ void write_tile(const float16v (&acc)[2][NT], T *__re
   }
 }
 
-// dst[rows[r]] += acc for the 64 rows of a wave (rows[] in LDS, -1 = none; no
+// dst[rows[r]] += acc for the MT * 32 rows of a wave (rows[] in LDS, -1 = none; no
 // atomics: the caller owns these rows).  All reads of the old values are issued
 // before the first add so that they overlap.
-template <typename T, int NT>
-__device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__restrict__ dst,
+template <typename T, int NT, int MT>
+__device__ __forceinline__ void add_rows(const float16v (&acc)[MT][NT], T *__restrict__ dst,
                                          const int *__restrict__ rows, int c_dst, int cd0,
                                          int lane) {
   const int h = lane / 32, col = lane % 32;
   if constexpr (sizeof(T) == 4) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       int row[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) row[r] = rows[mt * 32 + (r / 4) * 8 + h * 4 + (r % 4)];
@@ -138,7 +138,7 @@ __device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__rest
   } else {
     const bool odd = col & 1;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       int row[8];
 #pragma unroll
       for (int rp = 0; rp < 8; ++rp) {
@@ -174,20 +174,21 @@ __device__ __forceinline__ void add_rows(const float16v (&acc)[2][NT], T *__rest
 // R rows at a time, and come back row-major, so every lane adds 4 consecutive
 // columns of one row and a destination row is read and written as whole
 // 64..256-byte runs by neighbouring lanes instead of 4 bytes per lane.
-// stage: the wave's staging tile, 64 * 2*S * 16 bytes.
-template <typename T, int NT, int S, bool ATOMIC>
-__device__ __forceinline__ void add_rows_lds(const float16v (&acc)[2][NT], T *__restrict__ dst,
+// stage: the wave's staging tile, MT * 32 rows of 2*S * 16 bytes.
+template <typename T, int NT, int S, bool ATOMIC, int MT>
+__device__ __forceinline__ void add_rows_lds(const float16v (&acc)[MT][NT], T *__restrict__ dst,
                                              const int *__restrict__ rows, float *__restrict__ stage,
                                              int c_dst, int cd0, int lane) {
   constexpr int COLS = NT * 32;
-  constexpr int R = (64 * 2 * S * 16) / (COLS * 4) >= 32 ? 32 : (64 * 2 * S * 16) / (COLS * 4);
+  constexpr int WR = MT * 32;             // the wave's rows
+  constexpr int R = (WR * 2 * S * 16) / (COLS * 4) >= 32 ? 32 : (WR * 2 * S * 16) / (COLS * 4);
   if constexpr (R < 8) {
     if constexpr (ATOMIC) write_tile<T, NT, true>(acc, dst, rows, c_dst, cd0, lane);
     else add_rows<T, NT>(acc, dst, rows, c_dst, cd0, lane);
   } else {
     constexpr int CH = COLS / 4;            // 16-byte chunks per staged row
     constexpr int IT = R * CH / 64;         // chunks per lane and pass
-    constexpr int PASSES = 64 / R;
+    constexpr int PASSES = WR / R;
     const int h = lane / 32, col = lane % 32;
     // fp16 with up to 64 columns: the old values of ALL passes are fetched up front (the
     // registers of the gathered rows are free by now), so that the passes do not each wait

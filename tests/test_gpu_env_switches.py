@@ -81,3 +81,11 @@ def test_weights_re_laid_instead_of_read_as_they_lie():
     rules out the one-grid backward, whose input gradient reads them as they lie)."""
     names = run_child({"FGMS_RAW_WEIGHTS": "0"})
     assert "bwd_fused_kernel" not in names and "gms_rows_kernel(fwd)" in names, names
+
+
+def test_small_launches_on_256_row_tiles():
+    """FGMS_HALF_TILES=0: launches too small to fill the chip keep tiles of 256 rows instead of
+    128 (the test clouds are that small, so the default run above went through the 128-row
+    tiles and this one through the others; both meet the oracle)."""
+    names = run_child({"FGMS_HALF_TILES": "0"})
+    assert "bwd_fused_kernel" in names and "gms_rows_kernel(fwd)" in names, names
