@@ -269,24 +269,6 @@ def main():
             b_.copy_(a_)
         torch.cuda.synchronize()
         del a_, b_
-    # per-kernel durations: steps with a HIP event pair around every kernel launch (recorded on
-    # the launch stream by the library).  Kept out of the timed region below because the ten
-    # event records per step cost 20-30 us of stream time themselves; run first, so that they
-    # also bring the clocks up for runs that ask for few steps.
-    for _ in range(5):
-        step()
-    capi.profile_reset()
-    capi.profile_enable(True)
-    prof_steps = max(min(args.steps, 200), 50)
-    tp0 = time.perf_counter()
-    for _ in range(prof_steps):
-        step()
-    torch.cuda.synchronize()
-    tp1 = time.perf_counter()
-    capi.profile_enable(False)
-    recs = capi.profile_records()
-    capi.profile_reset()
-
     # gather-only pass over the rows the planned kernels read: the memory-side floor
     gather_floor = None
     if plan is not None and L["k_vol"] <= 64 and (L["c_in"] * D["in_feats"].element_size()) % 16 == 0 \
@@ -383,6 +365,29 @@ def main():
         for _ in range(5):
             other()
         surface_other = {"ms_per_step": timed(other, n_o), "steps": n_o}
+
+    # per-kernel durations: steps with a HIP event pair around every kernel launch (recorded on
+    # the launch stream by the library).  Kept out of the timed region below because the ten
+    # event records per step cost 20-30 us of stream time themselves.  It is the last of the
+    # measurement passes, right in front of the warm-up steps: the passes before it leave gaps
+    # (host work, synchronisations) after which the clocks take some 10 ms of load to come back
+    # up, more than the few warm-up steps a short run asks for (measured: 20 timed steps after 5
+    # warm-up steps 137-141 us per step coming from such a gap, 130.5-132.7 us behind 100 and
+    # more steps of load; 1000 timed steps 131 us).
+    for _ in range(5):
+        step()
+    capi.profile_reset()
+    capi.profile_enable(True)
+    prof_steps = max(min(args.steps, 200), 100)
+    tp0 = time.perf_counter()
+    for _ in range(prof_steps):
+        step()
+    torch.cuda.synchronize()
+    tp1 = time.perf_counter()
+    capi.profile_enable(False)
+    recs = capi.profile_records()
+    capi.profile_reset()
+
 
     # W warm-up steps, then the timed region: exactly K steps, nothing else on the stream
     for _ in range(args.warmup):
