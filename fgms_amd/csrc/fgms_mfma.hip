@@ -784,11 +784,12 @@ bool half_tiles_enabled() {
 // partial results does not depend on their order.  On launches that fill the chip the atomics
 // cost more than the split gains.)  The standalone and the one-grid backward launch share this
 // choice, so that their input gradients agree bit for bit; an input gradient takes the small
-// tiles only for long chains (24 stages and more), since in the backward launch its
-// workgroups share the chip with the weight gradient's and twice as many of them delay those.
-// Measured (MI355X, step = fwd + dgrad + wgrad): 32 -> 32 fp32 over 20 k voxels 64.0 -> 56.6 us,
-// 64 -> 128 fp16 stride-2 (49 k output rows) forward 21.5 -> 19.7 us; the 8-offset input
-// gradient of the transposed layer inside the backward launch 34.6 -> 35.9 us, hence the rule.
+// tiles only where they (times two, for the shared tiles) fill at most half of the slots, since
+// in the backward launch its workgroups share the chip with the weight gradient's and more of
+// them delay those.  Measured (MI355X, 64 -> 64 fp16 over 10 k / 20 k / 50 k / 60 k voxels of the
+// indoor cloud): forward 23.5 -> 16.9, 23.3 -> 18.3, 26.5 -> 22.8, 28.5 -> 25.7 us; backward
+// launch 22.5 -> 17.0, 26.1 -> 20.9, 35.6 -> 36.0, 43.2 -> 47.8 us (128 -> 128 over 28 k voxels:
+// 53.2 -> 63.0 us), hence the rule; 32 -> 32 fp32 over 20 k voxels, whole step: 64.0 -> 56.6 us.
 struct RowsGrid {
   bool half_tiles;
   unsigned gx, gz;
@@ -797,9 +798,9 @@ struct RowsGrid {
 RowsGrid rows_grid(int64_t n_dst, unsigned gy, int stages, bool can_half, bool has_table, int table_grid,
                    bool pair_view, int wgs_per_cu, bool input_gradient) {
   RowsGrid g{};
+  const int64_t small_tiles = (int64_t)((n_dst + 127) / 128) * gy;
   g.half_tiles = can_half && half_tiles_enabled() && !has_table && !pair_view &&
-                 (!input_gradient || stages >= 24) &&
-                 (int64_t)((n_dst + 127) / 128) * gy <= (int64_t)num_cus() * 4;
+                 (input_gradient ? small_tiles * 4 <= (int64_t)num_cus() * 3 : small_tiles <= (int64_t)num_cus() * 4);
   const int tile_rows = g.half_tiles ? kTileRows / 2 : kTileRows;
   g.gx = has_table ? (unsigned)table_grid : (unsigned)((n_dst + tile_rows - 1) / tile_rows);
   const int64_t slots = (int64_t)num_cus() * (g.half_tiles ? 4 : wgs_per_cu);
