@@ -792,6 +792,7 @@ bool half_tiles_enabled() {
 // 53.2 -> 63.0 us), hence the rule; 32 -> 32 fp32 over 20 k voxels, whole step: 64.0 -> 56.6 us.
 struct RowsGrid {
   bool half_tiles;
+  bool drop_table;      // the launch does better on plain 128-row tiles than on the plan's tile table
   unsigned gx, gz;
   int part_stages;
 };
@@ -799,6 +800,14 @@ RowsGrid rows_grid(int64_t n_dst, unsigned gy, int stages, bool can_half, bool h
                    bool pair_view, int wgs_per_cu, bool input_gradient) {
   RowsGrid g{};
   const int64_t small_tiles = (int64_t)((n_dst + 127) / 128) * gy;
+  // A forward launch of 1.25 to 3 workgroups of 256 rows per CU is neither alone on its CUs nor
+  // a full round: 128-row tiles in plain order then beat the table's XCD-aware 256-row tiles
+  // (64 -> 64 fp16 over 100 k / 130 k voxels: 40.9 -> 34.4, 41.2 -> 36.9 us; 70 k voxels, 1.07 per
+  // CU: 28.5 us with the table against 32.4).
+  g.drop_table = can_half && half_tiles_enabled() && has_table && !pair_view && !input_gradient &&
+                 small_tiles <= (int64_t)num_cus() * 4 &&
+                 (int64_t)((n_dst + 255) / 256) * gy * 4 >= (int64_t)num_cus() * 5;
+  if (g.drop_table) has_table = false;
   g.half_tiles = can_half && half_tiles_enabled() && !has_table && !pair_view &&
                  (input_gradient ? small_tiles * 4 <= (int64_t)num_cus() * 3 : small_tiles <= (int64_t)num_cus() * 4);
   const int tile_rows = g.half_tiles ? kTileRows / 2 : kTileRows;
@@ -861,6 +870,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   const RowsGrid rg = rows_grid(a.n_dst, gy, a.k_vol * slabs, kCanHalf, tile_order != nullptr, tile_grid, pair_view,
                                 NT == 4 ? 2 : 3, a.transpose_w);
   const bool half_tiles = rg.half_tiles;
+  if (rg.drop_table) tile_order = nullptr;
   const size_t lds_rows = half_tiles ? s.lds_rows_bytes - (size_t)kWaves * 32 * (2 * S * 16 + 2 * sizeof(int))
                                      : s.lds_rows_bytes;
   const unsigned gx = rg.gx;

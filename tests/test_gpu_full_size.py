@@ -208,3 +208,31 @@ def test_backward_in_one_launch_full_size(capi, oracle, shape, dtype):
     capi.profile_reset()
     plan.close()
     assert names == {"bwd_fused_kernel"}, names
+
+
+@pytest.mark.parametrize("voxels", [9000, 30000, 62000, 70000, 100000, 128000, 140000])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32], ids=["fp16", "fp32"])
+def test_every_grid_choice_against_oracle(capi, oracle, voxels, dtype):
+    """The output-stationary launch picks its grid by the number of rows: tiles of 128 rows
+    shared by two workgroups (9 k, 30 k), tiles of 128 rows (62 k), the plan's tile table with
+    256-row tiles (70 k: about one workgroup per CU), plain 128-row tiles although a table
+    exists (100 k, 128 k: forward only), the table again (140 k and up).  Forward, input and
+    weight gradient of a 64 -> 64 layer against the oracle at each size, the input gradient of
+    the one-grid backward call bit for bit equal to the separate call's."""
+    rng = np.random.default_rng(91)
+    vox = clouds.cloud_indoor(clouds.rng_for(2), target=voxels)
+    L = clouds.submanifold_case(vox, 64, 64, dtype, rng)
+    D = G.to_dev(L)
+    capi.set_kernel_policy(4)      # the kernels with a plan, whatever the cloud's row-slot fill
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    mode = G.mode_of(L["in_feats"].dtype, False)
+    a = (L["knnz"], L["imap"], L["omap"])
+    out = G.run_fwd(capi, D, fused=True, plan=plan)
+    G.assert_close(out, oracle.c_fwd(L["in_feats"], L["kernel"], *a, L["n_out"]), mode, "fwd")
+    gi_s, _ = G.run_bwd(capi, D, plan=plan, split=True)
+    gi, gw = G.run_bwd(capi, D, plan=plan)
+    capi.set_kernel_policy(0)
+    plan.close()
+    assert np.array_equal(gi, gi_s)
+    G.assert_close(gi, oracle.c_dgrad(L["out_grad"], L["kernel"], *a, L["n_in"]), mode, "dgrad")
+    G.assert_close(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *a, L["k_vol"]), mode, "wgrad")
