@@ -800,13 +800,13 @@ RowsGrid rows_grid(int64_t n_dst, unsigned gy, int stages, bool can_half, bool h
                    bool pair_view, int wgs_per_cu, bool input_gradient) {
   RowsGrid g{};
   const int64_t small_tiles = (int64_t)((n_dst + 127) / 128) * gy;
-  // A forward launch of 1.25 to 3 workgroups of 256 rows per CU is neither alone on its CUs nor
-  // a full round: 128-row tiles in plain order then beat the table's XCD-aware 256-row tiles
-  // (64 -> 64 fp16 over 100 k / 130 k voxels: 40.9 -> 34.4, 41.2 -> 36.9 us; 70 k voxels, 1.07 per
-  // CU: 28.5 us with the table against 32.4).
+  // A forward launch too big to share its 256-row tiles between two workgroups (below) and
+  // not yet a full round of them is neither short-chained nor busy: 128-row tiles in plain order
+  // then beat the table's XCD-aware 256-row tiles (64 -> 64 fp16 over 100 k / 130 k voxels:
+  // 40.9 -> 34.4, 41.2 -> 36.9 us; 70 k / 80 k voxels with shared 256-row tiles: 28.1 / 29.1 us).
   g.drop_table = can_half && half_tiles_enabled() && has_table && !pair_view && !input_gradient &&
                  small_tiles <= (int64_t)num_cus() * 4 &&
-                 (int64_t)((n_dst + 255) / 256) * gy * 4 >= (int64_t)num_cus() * 5;
+                 ((int64_t)table_grid * gy * 2 > (int64_t)num_cus() * wgs_per_cu || stages < 8);
   if (g.drop_table) has_table = false;
   g.half_tiles = can_half && half_tiles_enabled() && !has_table && !pair_view &&
                  (input_gradient ? small_tiles * 4 <= (int64_t)num_cus() * 3 : small_tiles <= (int64_t)num_cus() * 4);

@@ -214,9 +214,9 @@ def test_backward_in_one_launch_full_size(capi, oracle, shape, dtype):
 @pytest.mark.parametrize("dtype", [np.float16, np.float32], ids=["fp16", "fp32"])
 def test_every_grid_choice_against_oracle(capi, oracle, voxels, dtype):
     """The output-stationary launch picks its grid by the number of rows: tiles of 128 rows
-    shared by two workgroups (9 k, 30 k), tiles of 128 rows (62 k), the plan's tile table with
-    256-row tiles (70 k: about one workgroup per CU), plain 128-row tiles although a table
-    exists (100 k, 128 k: forward only), the table again (140 k and up).  Forward, input and
+    shared by two workgroups (9 k, 30 k, 62 k), the plan's tile table with 256-row tiles shared
+    by two workgroups (70 k), plain 128-row tiles although a table exists (100 k, 128 k:
+    forward only), the table again (140 k and up).  Forward, input and
     weight gradient of a 64 -> 64 layer against the oracle at each size, the input gradient of
     the one-grid backward call bit for bit equal to the separate call's."""
     rng = np.random.default_rng(91)
