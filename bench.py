@@ -116,9 +116,11 @@ def cpu_baseline(name, budget_s=12.0):
     want = min(1.0, scale * budget_s / max(dt, 1e-3))
     repeats = 1
     if want > 1.2 * scale:
-        # the full cloud costs dt / scale per repeat; repeat it to fill the budget
-        repeats = max(1, min(200, int(budget_s / max(dt / scale * want, 1e-3))))
+        # two passes at the sample's size tell what a repeat costs (the small probe also pays for
+        # the thread pool's start and first-touch page faults); then as many as fill the budget
         scale = want
+        dt, flops, L = run(scale, 2)
+        repeats = max(1, min(200, int(budget_s / max(dt / 2, 1e-3))))
         dt, flops, L = run(scale, repeats)
     # one thread, on a sample a sixteenth of that (about the same time again at most)
     dt1, flops1, L1 = run(max(scale / 16.0, 0.01), 1, threads=1)
