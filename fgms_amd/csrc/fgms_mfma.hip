@@ -812,7 +812,11 @@ RowsGrid rows_grid(int64_t n_dst, unsigned gy, int stages, bool can_half, bool h
                  (input_gradient ? small_tiles * 4 <= (int64_t)num_cus() * 3 : small_tiles <= (int64_t)num_cus() * 4);
   const int tile_rows = g.half_tiles ? kTileRows / 2 : kTileRows;
   g.gx = has_table ? (unsigned)table_grid : (unsigned)((n_dst + tile_rows - 1) / tile_rows);
-  const int64_t slots = (int64_t)num_cus() * (g.half_tiles ? 4 : wgs_per_cu);
+  // (an input gradient shares its launch with the weight gradient: its 256-row tiles are shared
+  // only up to 2.25 workgroups per CU; 64 -> 64 fp16 backward launch over 70 k / 80 k / 90 k voxels
+  // shared 50.7 / 58.6 / 60.4 us, not shared 54.7 / 55.8 / 56.4 us)
+  const int64_t slots = g.half_tiles ? (int64_t)num_cus() * 4
+                        : input_gradient ? (int64_t)num_cus() * 9 / 4 : (int64_t)num_cus() * wgs_per_cu;
   g.gz = 1;
   g.part_stages = 1;
   if (!pair_view && (int64_t)g.gx * gy * 2 <= slots && stages >= 8) {
