@@ -647,18 +647,22 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
     set_error("fgms_plan_create: pinned flag block / event creation failed");
     return fail(FGMS_E_NOMEM);
   }
-  // weight-gradient row bands: about 2048 output rows each but enough bands to
-  // fill the chip (bands x offsets >= ~1536 workgroups) and no more than leaves a
-  // workgroup ~400 pairs on average; a multiple of 8 (one per XCD), 8..kMaxBands
+  // weight-gradient row bands: 8, 16, 32 or 64 (the XCDs take them in groups of 1, 2, 4 or 8;
+  // other counts measured worse), the fewest that leave an (offset, band) cell at most ~1 900
+  // pairs -- a workgroup's fixed costs (first loads, the four waves' partial tiles summed through
+  // LDS, 16 KB of atomic updates) are those of ~600 pairs, and with bigger cells the chip waits
+  // for the last ones -- then more while the cells are fewer than 1.5 per CU and keep ~400 pairs.
+  // 64 -> 64 fp16 backward launch with 64 bands throughout / with this rule: 50 k voxels 35.5 /
+  // 29.8 us, 80 k 55.6 / 45.2, 100 k 59.1 / 46.2, 120 k 61.5 / 55.6, 140 k 67.7 / 65.3 (32 bands
+  // each), 170 k and 200 k voxels 64 bands either way.
   {
-    int64_t want = n_out / 2048;
-    const int64_t fill = (1536 + k_vol - 1) / k_vol;
-    if (want < fill) want = fill;
-    const int64_t by_work = n_pairs / ((int64_t)k_vol * 384);
-    if (want > by_work) want = by_work;
-    want = (want + 7) / 8 * 8;
     constexpr int kMaxBands = 64;
-    p->band_count = (int)(want < 8 ? 8 : (want > kMaxBands ? kMaxBands : want));
+    int bands = 8;
+    while (bands < kMaxBands && n_pairs / ((int64_t)k_vol * bands) > 1900) bands *= 2;
+    while (bands < kMaxBands && (int64_t)bands * k_vol * 2 < 3 * (int64_t)num_cus() &&
+           n_pairs / ((int64_t)k_vol * bands * 2) >= 384)
+      bands *= 2;
+    p->band_count = bands;
   }
   const int band_rows = (int)((n_out + p->band_count - 1) / p->band_count);
   p->band_rows = band_rows;
