@@ -278,46 +278,38 @@ __device__ __forceinline__ void wgrad_wave_body(
     st += 4;
   }
 
-  // sum the four waves' tiles: (2, 3) -> (0, 1), then 1 -> 0, through LDS
+  // Sum the four waves' tiles through LDS and flush.  Every wave ends up with a quarter of the
+  // summed tile (accumulator registers q * R / 4 ... of the R = BI * BJ * 16 a lane holds) and
+  // flushes that: one barrier, and the atomic updates of the tile issued by four waves instead
+  // of one.  red: [quarter][contribution 0..2][register of the quarter][lane].
   float *red = reinterpret_cast<float *>(lds);
-  constexpr int kTileFloats = BI * BJ * 16 * 64;
-  auto put = [&](int slot) {
+  constexpr int R = BI * BJ * 16, RQ = R / 4;
+  __syncthreads();                  // every wave is done with its staging tiles
 #pragma unroll
-    for (int ti = 0; ti < BI; ++ti)
+  for (int q = 0; q < 4; ++q) {
+    if (q == wave) continue;
+    const int slot = wave < q ? wave : wave - 1;
 #pragma unroll
-      for (int tj = 0; tj < BJ; ++tj)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          red[(size_t)slot * kTileFloats + ((ti * BJ + tj) * 16 + r) * 64 + lane] = acc[ti][tj][r];
-  };
-  auto take = [&](int slot) {
-#pragma unroll
-    for (int ti = 0; ti < BI; ++ti)
-#pragma unroll
-      for (int tj = 0; tj < BJ; ++tj)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          acc[ti][tj][r] += red[(size_t)slot * kTileFloats + ((ti * BJ + tj) * 16 + r) * 64 + lane];
-  };
+    for (int j = 0; j < RQ; ++j) {
+      const int idx = q * RQ + j, t = idx / 16;
+      red[(size_t)((q * 3 + slot) * RQ + j) * 64 + lane] = acc[t / BJ][t % BJ][idx % 16];
+    }
+  }
   __syncthreads();
-  if (wave >= 2) put(wave - 2);
-  __syncthreads();
-  if (wave < 2) take(wave);
-  __syncthreads();
-  if (wave == 1) put(0);
-  __syncthreads();
-  if (wave != 0) return;
-  take(0);
   const int h = lane >> 5, c = lane & 31;
 #pragma unroll
-  for (int ti = 0; ti < BI; ++ti)
+  for (int q = 0; q < 4; ++q) {
+    if (q != wave) continue;
 #pragma unroll
-    for (int tj = 0; tj < BJ; ++tj) {
-      float *tile = gw32 + ((size_t)k * c_in + ci0 + ti * 32) * c_out + co0 + tj * 32 + c;
+    for (int j = 0; j < RQ; ++j) {
+      const int idx = q * RQ + j, t = idx / 16, r = idx % 16, ti = t / BJ, tj = t % BJ;
+      float v = acc[ti][tj][r];
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        atomic_add(tile + (size_t)((r / 4) * 8 + h * 4 + (r % 4)) * c_out, acc[ti][tj][r]);
+      for (int slot = 0; slot < 3; ++slot) v += red[(size_t)((q * 3 + slot) * RQ + j) * 64 + lane];
+      // accumulator register r of lane l is row (r/4)*8 + (l/32)*4 + r%4, column l%32 of its 32 x 32 tile
+      atomic_add(gw32 + ((size_t)k * c_in + ci0 + ti * 32 + (r / 4) * 8 + h * 4 + (r % 4)) * c_out + co0 + tj * 32 + c, v);
     }
+  }
 }
 
 
