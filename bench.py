@@ -179,9 +179,6 @@ def main():
     ap.add_argument("--surface", default="cabi", choices=["cabi", "backend"],
                     help="what `value` times: the C ABI with an explicit plan (default) or the python "
                          "extension FGMS.backend (plan from its cache); the other one is reported next to it")
-    ap.add_argument("--coords-plan", action="store_true",
-                    help="build the plan with the voxel coordinates (fgms_plan_create_coords) and run the "
-                         "LDS-neighbourhood kernel where it applies (kernel policy 6)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run plain 256 MiB device copies (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -198,24 +195,12 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     L, passes, arch80 = make_case(args.workload, args.scale)
     D = to_dev(L)
-    if args.coords_plan:
-        args.policy = 6
     capi.set_kernel_policy(args.policy)
     backend.fgms_set_kernel_policy(args.policy)
     backend.fgms_plan_cache(not args.no_plan)
-    coords = None
-    if args.coords_plan:
-        import numpy as np
-        from fgms_amd import clouds
-        if WORKLOADS[args.workload][0] != 2 and not args.workload.startswith("cfg5-skinny"):
-            print("bench.py: --coords-plan is wired for the submanifold layers over the indoor cloud", file=sys.stderr)
-            sys.exit(2)
-        coords = torch.from_numpy(np.ascontiguousarray(
-            clouds.cloud_indoor(clouds.rng_for(2), target=int(200000 * args.scale)), dtype=np.int32)).cuda()
 
     def make_plan():
-        return capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"],
-                         in_coords=coords, out_coords=coords, coord_bits=9 if coords is not None else 0)
+        return capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
 
     plan = None if args.no_plan else make_plan()
     dt = D["in_feats"].dtype
@@ -254,7 +239,7 @@ def main():
         print("bench.py: FGMS.backend has no entry point for one gradient alone", file=sys.stderr)
         sys.exit(2)
     step = step_backend if args.surface == "backend" else step_cabi
-    other = step_cabi if args.surface == "backend" else (step_backend if backend_ok and coords is None else None)
+    other = step_cabi if args.surface == "backend" else (step_backend if backend_ok else None)
 
     def timed(fn, n):
         torch.cuda.synchronize()
@@ -475,7 +460,6 @@ def main():
         "config": {"workload": args.workload, "voxels_in": L["n_in"], "voxels_out": L["n_out"],
                    "pairs": m, "k_vol": L["k_vol"], "c_in": L["c_in"], "c_out": L["c_out"],
                    "plan": plan is not None, "policy": args.policy, "surface": args.surface,
-                   "plan_with_coordinates": coords is not None,
                    "row_slots_per_pair": (round(plan.stats()["blocks_fwd"] * 64.0 / max(plan.stats()["pairs"], 1), 3)
                                           if plan is not None else None)},
         "kernels": kernels,

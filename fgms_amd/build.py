@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libfgms_hip.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
 HIP_SOURCES = ["fgms_api.hip", "fgms_generic.hip", "fgms_plan.hip", "fgms_mfma.hip", "fgms_small.hip", "fgms_wgrad.hip",
-               "fgms_probe.hip", "fgms_kmap.hip", "fgms_halo.hip", "fgms_wide.hip"]
+               "fgms_probe.hip", "fgms_kmap.hip", "fgms_wide.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXX = os.environ.get("CXX", "g++")
@@ -106,19 +106,6 @@ def build_cabi_demo(verbose=False):
     return DEMO_PATH
 
 
-PROBES_PATH = os.path.join(LIB_DIR, "machine_probes")
-
-
-def build_machine_probes(verbose=False):
-    """csrc/machine_probes.hip: stand-alone micro-benchmarks of the machine limits the kernels
-    run into (atomics, row gathers, direct-to-LDS loads, LDS access patterns)."""
-    o = _run([HIPCC] + [f for f in HIP_FLAGS if f != "-fPIC"] +
-             [os.path.join(CSRC, "machine_probes.hip"), "-o", PROBES_PATH])
-    if verbose and o.strip():
-        print(o)
-    return PROBES_PATH
-
-
 def up_to_date():
     """True when both shared objects exist and are newer than every source and header."""
     outs = [LIB_PATH, torch_ext_path()]
@@ -136,7 +123,6 @@ def build_all(verbose=False, force=True):
     build_hip_lib(verbose)
     build_torch_ext(verbose)
     build_cabi_demo(verbose)
-    build_machine_probes(verbose)
 
 
 if __name__ == "__main__":

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfgms_hip.so")
 
 F32, F16 = 0, 1
 SYMBOLS = [
-    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_create_coords", "fgms_plan_transposed", "fgms_plan_destroy",
+    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_transposed", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_plan_stats", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_wgrad_static", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
     "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map",
@@ -39,7 +39,6 @@ def lib():
     L.fgms_version.restype = ctypes.c_char_p
     L.fgms_last_error.restype = ctypes.c_char_p
     L.fgms_plan_create.argtypes = [ctypes.POINTER(vp), vp, vp, vp, i64, i64, i32, i64, vp]
-    L.fgms_plan_create_coords.argtypes = [ctypes.POINTER(vp), vp, vp, vp, i64, i64, i32, i64, vp, vp, i32, vp]
     L.fgms_plan_transposed.argtypes = [ctypes.POINTER(vp), vp]
     L.fgms_plan_destroy.argtypes = [vp]
     L.fgms_plan_destroy.restype = None
@@ -133,28 +132,14 @@ def profile_records():
 class Plan:
     """Neighbour tables for one kernel map (``fgms_plan_create``)."""
 
-    def __init__(self, kpos, in_map, out_map, n_in, n_out, in_coords=None, out_coords=None, coord_bits=0):
-        """in_coords / out_coords (int32 [n, 3] on the GPU, optional): the rows' voxel
-        coordinates; with them the plan orders the rows along a Morton curve
-        (``fgms_plan_create_coords``)."""
+    def __init__(self, kpos, in_map, out_map, n_in, n_out):
         for t, n in ((kpos, "kpos"), (in_map, "in_map"), (out_map, "out_map")):
             _need(t, n, torch.int32)
         self._keep = (kpos, in_map, out_map)
         self._h = ctypes.c_void_p()
-        if in_coords is None and out_coords is None:
-            _check(lib().fgms_plan_create(ctypes.byref(self._h), _p(kpos), _p(in_map), _p(out_map),
-                                          int(n_in), int(n_out), kpos.numel() - 1, in_map.numel(),
-                                          _stream()))
-            return
-        if in_coords is None or out_coords is None:
-            raise ValueError("pass the coordinates of both sides (the same tensor for a submanifold map)")
-        for t, n, rows in ((in_coords, "in_coords", n_in), (out_coords, "out_coords", n_out)):
-            _need(t, n, torch.int32)
-            if t.dim() != 2 or t.shape[0] != rows or t.shape[1] != 3:
-                raise ValueError("%s must be [%d, 3]" % (n, rows))
-        _check(lib().fgms_plan_create_coords(ctypes.byref(self._h), _p(kpos), _p(in_map), _p(out_map),
-                                             int(n_in), int(n_out), kpos.numel() - 1, in_map.numel(),
-                                             _p(in_coords), _p(out_coords), int(coord_bits), _stream()))
+        _check(lib().fgms_plan_create(ctypes.byref(self._h), _p(kpos), _p(in_map), _p(out_map),
+                                      int(n_in), int(n_out), kpos.numel() - 1, in_map.numel(),
+                                      _stream()))
 
     @property
     def handle(self):

@@ -292,7 +292,7 @@ bool sparse_rows(const GmsArgs &a, const Plan *plan) {
   return slots_per_pair > (need > 1.4 ? need : 1.4);
 }
 
-enum class Route { kSkinny, kHalo, kRows, kPairView, kWide, kPairs, kGeneric };
+enum class Route { kSkinny, kRows, kPairView, kWide, kPairs, kGeneric };
 
 // Which kernel a forward / input-gradient pass takes.
 Route route_of(const GmsArgs &a, const Plan *plan) {
@@ -301,9 +301,6 @@ Route route_of(const GmsArgs &a, const Plan *plan) {
   const bool pair_view = !dense && pair_view_gms_supported(a, plan);
   if (g_policy == 5 && pair_view) return Route::kPairView;
   if (!dense && (g_policy == 0 || g_policy == 4) && small_gms_supported(a, plan)) return Route::kSkinny;
-  // the kernel that keeps a tile's neighbourhood rows in LDS: on request only (it measures
-  // slower than the output-stationary kernel that gathers per pair, see fgms_halo.hip)
-  if (!dense && g_policy == 6 && halo_gms_supported(a, plan)) return Route::kHalo;
   if (g_policy == 7 && wide_gms_supported(a)) return Route::kWide;
   if (!dense && g_policy != 2 && planned_gms_supported(a, plan) &&
       !(g_policy != 4 && sparse_rows(a, plan) && mfma_gms_supported(a)))
@@ -346,7 +343,6 @@ int run_gms_one(GmsArgs a, const Plan *plan) {
   if ((!dense && a.n_pairs == 0) || (dense && a.n_dense == 0)) return FGMS_OK;
   switch (route_of(a, plan)) {
     case Route::kSkinny: return launch_small_gms(a, plan);
-    case Route::kHalo: return launch_halo_gms(a, plan);
     case Route::kRows: return launch_planned_gms(a, plan);
     case Route::kPairView: return launch_pair_view_gms(a, plan);
     case Route::kWide: return launch_wide_gms(a);

@@ -96,19 +96,6 @@ struct WgradArgs {
   float *acc_override;
 };
 
-// One direction of a plan's tile tables for the kernels that keep a tile's neighbourhood in
-// LDS (fgms_halo.hip): destination rows in a spatially compact order, cut into tiles of 128.
-struct HaloSide {
-  int32_t *order;               // [n_tiles * 128] position -> destination row, -1 = padding
-  int32_t *rows;                // [n_tiles][list_cap] the tile's distinct source rows, in source order (padded to 8s)
-  int32_t *count;               // [n_tiles] how many
-  unsigned short *lnbr;         // [n_tiles][k_vol][32][4] index into the tile's list by (row of block, block), 0xFFFF = no neighbour
-  unsigned long long *mask32;   // [n_tiles * 4] offsets in use per block of 32 positions
-  int n_tiles, list_cap;
-  int64_t extra_rounds;         // sum over tiles of the LDS rounds beyond the first
-  bool ok;                      // built and every tile's list fitted list_cap
-};
-
 constexpr int kPlanFlags = 13;      // ints the plan build reports back (see fgms_plan.hip)
 
 // Plan: neighbour tables built from the pair lists.
@@ -181,7 +168,6 @@ struct Plan {
   int32_t *pv_in, *pv_out;        // [pv_rows]
   unsigned long long *pv_mask;    // [pv_rows / 64]
   int64_t pv_rows;                // a multiple of 256
-  HaloSide halo[2];   // [0] forward (destination = output rows), [1] input gradient
   bool fwd_ok;        // no offset maps two pairs onto one output row
   bool dgrad_ok;      // no offset maps two pairs from one input row
 };
@@ -242,11 +228,6 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p);
 // The same kernel over the plan's pair view (no wasted row slots, atomic adds).
 bool pair_view_gms_supported(const GmsArgs &a, const Plan *p);
 int launch_pair_view_gms(const GmsArgs &a, const Plan *p);
-// Tile tables of the LDS-neighbourhood kernels (fgms_halo.hip).
-int halo_morton_order(const int32_t *coords, int64_t n, int coord_bits, int32_t **order, int32_t **inv,
-                      std::vector<void *> *tmp, hipStream_t s);
-int halo_build(Plan *p, int d, const int32_t *nbr_by_pos, const int32_t *plan_pos, const int32_t *order_dst,
-               const int32_t *inv_src, const int32_t *order_src, int *flags, hipStream_t s);
 // Notes that a launch on `stream` reads the plan.
 inline void plan_touch(const Plan *p, hipStream_t stream) {
   if (p->last_stream != stream && p->resolved) p->many_streams = true;
@@ -254,9 +235,6 @@ inline void plan_touch(const Plan *p, hipStream_t stream) {
 }
 // The plan with its build results known, or nullptr (see fgms_plan.hip).
 const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc);
-void halo_release(Plan *p);
-bool halo_gms_supported(const GmsArgs &a, const Plan *p);
-int launch_halo_gms(const GmsArgs &a, const Plan *p);
 int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
                      const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
                      int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,

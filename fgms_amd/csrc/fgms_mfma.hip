@@ -84,6 +84,30 @@ template <typename T, int NT, int S, int MT>
 __device__ __forceinline__ void mma_slab(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                          const int4v *__restrict__ w_lds, int slab, int lane) {
   const int h = lane / 32, r = lane % 32;
+  if constexpr (sizeof(T) == 2 && NT <= 2) {
+    // (pipelined like mma_slab_raw below: the next k-step's fragments are requested first)
+    int4v a[2][MT], b[2][NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) b[0][nt] = w_lds[((slab * S) * NT + nt) * 64 + lane];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) a[0][mt] = a_lds[a_slot<S>(mt * 32 + r, h * S)];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      if (s + 1 < S) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) b[(s + 1) & 1][nt] = w_lds[((slab * S + s + 1) * NT + nt) * 64 + lane];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) a[(s + 1) & 1][mt] = a_lds[a_slot<S>(mt * 32 + r, h * S + s + 1)];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a[s & 1][mt], b[s & 1][nt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    return;
+  }
 #pragma unroll
   for (int s = 0; s < S; ++s) {
     int4v b[NT];
@@ -98,22 +122,35 @@ __device__ __forceinline__ void mma_slab(float16v (&acc)[MT][NT], const int4v *_
   }
 }
 
+// The MFMA phase of a stage, software-pipelined by hand: the fragments of k-step s + 1 are
+// requested from LDS before the MFMAs of k-step s are issued (two sets of fragment registers),
+// so that a wave's matrix instructions follow each other instead of each pair waiting out an
+// LDS round trip.  The scheduling barriers keep the compiler from sinking the reads back to
+// their uses (left alone it emits read, wait, two MFMAs, read, wait, ... in source order).
 // acc[mt][nt] += A(slab) x W(slab), weights as raw_weight_frag reads them.
 template <typename T, int NT, int S, int MT>
 __device__ __forceinline__ void mma_slab_raw(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                              const int4v *__restrict__ w_lds, int lane) {
   const int h = lane / 32, r = lane % 32;
+  int4v a[2][MT], b[2][NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) b[0][nt] = raw_weight_frag<NT, S>(w_lds, 0, nt, lane);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) a[0][mt] = a_lds[a_slot<S>(mt * 32 + r, h * S)];
 #pragma unroll
   for (int s = 0; s < S; ++s) {
-    int4v b[NT];
+    if (s + 1 < S) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) b[nt] = raw_weight_frag<NT, S>(w_lds, s, nt, lane);
+      for (int nt = 0; nt < NT; ++nt) b[(s + 1) & 1][nt] = raw_weight_frag<NT, S>(w_lds, s + 1, nt, lane);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+      for (int mt = 0; mt < MT; ++mt) a[(s + 1) & 1][mt] = a_lds[a_slot<S>(mt * 32 + r, h * S + s + 1)];
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a[s & 1][mt], b[s & 1][nt]);
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -127,17 +164,41 @@ template <typename T, int NT, int S, int MT>
 __device__ __forceinline__ void mma_slab_rawt(float16v (&acc)[MT][NT], const int4v *__restrict__ a_lds,
                                               const int4v *__restrict__ w_lds, int lane) {
   const int h = lane / 32, r = lane % 32;
+  if constexpr (sizeof(T) == 4) {
+    // (fp32: a k-step is sixteen MFMAs of 64 cycles, long enough to cover the next reads)
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      int4v b[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[a_slot<S>(nt * 32 + r, h * S + s)];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+      }
+    }
+    return;
+  }
+  int4v a[2][MT], b[2][NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) b[0][nt] = w_lds[a_slot<S>(nt * 32 + r, h * S)];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) a[0][mt] = a_lds[a_slot<S>(mt * 32 + r, h * S)];
 #pragma unroll
   for (int s = 0; s < S; ++s) {
-    int4v b[NT];
+    if (s + 1 < S) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) b[nt] = w_lds[a_slot<S>(nt * 32 + r, h * S + s)];
+      for (int nt = 0; nt < NT; ++nt) b[(s + 1) & 1][nt] = w_lds[a_slot<S>(nt * 32 + r, h * S + s + 1)];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+      for (int mt = 0; mt < MT; ++mt) a[(s + 1) & 1][mt] = a_lds[a_slot<S>(mt * 32 + r, h * S + s + 1)];
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a[s & 1][mt], b[s & 1][nt]);
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -310,6 +371,61 @@ __device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (
   }
 }
 
+// The same two steps for the output-stationary kernel, through buffer loads: `offs` holds a
+// BYTE offset per row of the wave's tile (row index x row bytes), kAbsentRow for a row that has
+// no neighbour through this offset.  The buffer's range check turns every load at or beyond
+// `src_bytes` into zeros, so an absent row arrives as zeros by itself: no select on the way to
+// LDS, no row index kept per load, 32-bit address arithmetic.  (src_bytes < 2^31, checked by
+// the host, keeps kAbsentRow + any offset inside a row from wrapping round.)
+constexpr unsigned kAbsentRow = 0x80000000u;
+constexpr size_t kMaxBufferBytes = 0x7fff0000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_resource(const void *base, unsigned bytes) {
+  // raw buffer: stride 0, num_records in bytes, 32-bit data format
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+template <int S, int N>
+__device__ __forceinline__ void gather_issue_buf(int4v (&v)[N], const unsigned *__restrict__ offs,
+                                                 __amdgpu_buffer_rsrc_t rsrc, int slab, int lane) {
+  constexpr int C = 2 * S;
+  unsigned off[N];
+#pragma unroll
+  for (int it = 0; it < N; ++it) off[it] = offs[(it * 64 + lane) / C] + (unsigned)((lane % C) * 16);
+#pragma unroll
+  for (int it = 0; it < N; ++it)
+    v[it] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off[it], slab * (C * 16), 0));
+}
+
+template <int S, int N>
+__device__ __forceinline__ void gather_commit_buf(int4v *__restrict__ a_lds, const int4v (&v)[N], int lane) {
+  constexpr int C = 2 * S;
+  if constexpr (C == 8) {
+    // a_slot(it * 8 + lane / 8, lane % 8) spelled out: the swizzle term (row >> 1) & 7 is
+    // lane / 16 for even `it` and lane / 16 + 4 for odd ones, so two per-lane bases and
+    // immediate offsets address all N writes
+    const int base = (lane / 8) * 8, c = lane % 8, x = lane / 16;
+    const int even = base + (c ^ x), odd = base + (c ^ (x + 4));
+#pragma unroll
+    for (int it = 0; it < N; ++it) a_lds[((it & 1) ? odd : even) + it * 64] = v[it];
+  } else {
+#pragma unroll
+    for (int it = 0; it < N; ++it) {
+      const int slot = it * 64 + lane;
+      a_lds[a_slot<S>(slot / C, slot % C)] = v[it];
+    }
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void gather_commit_bf3_buf(int4v *__restrict__ a_lds, const int4v (&v)[N], int lane) {
+#pragma unroll
+  for (int it = 0; it < N; ++it) {
+    const int slot = it * 64 + lane;
+    split_and_store(a_lds, __builtin_bit_cast(float4v, v[it]), slot / 8, slot % 8, lane);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Pair-stationary kernel.
 // SPLIT: fp32 tensors whose caller allows tf32 precision, products in split bf16 (see
@@ -415,9 +531,17 @@ __device__ __forceinline__ void gms_rows_body(
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
     int c_src, int c_dst, int part_stages, int block_x, int block_y, int block_z, int grid_z,
-    int pair_view = 0) {
+    unsigned src_bytes, int pair_view = 0) {
   constexpr int E = Elem<T>::per_chunk;
   constexpr int C = 2 * S;
+  // 16-bit matrix instructions (fp16 tensors, fp32 tensors in split bf16): rows and weights come
+  // through buffer loads and the MFMA phase is pipelined by hand; plain fp32, whose MFMA phase is
+  // eight times as long, keeps pointer loads and interleaves them with its MFMAs instead
+  constexpr bool kBuf = sizeof(T) == 2 || RAW == 3 || RAW == 4;
+  const __amdgpu_buffer_rsrc_t rsrc = rows_resource(src, src_bytes);
+  const unsigned row_bytes = (unsigned)c_src * (unsigned)sizeof(T);
+  // byte offset of source row g in the buffer (kAbsentRow: no neighbour, the loads return zeros)
+  auto row_offset = [&](int g) { return !kBuf ? (unsigned)g : g < 0 ? kAbsentRow : (unsigned)g * row_bytes; };
   // pair view: `nbr` is one list of source rows for all offsets (a 64-row block belongs to
   // the one offset its mask names), `perm` the destination rows; results are added atomically
   const size_t nbr_stride = pair_view ? 0 : (size_t)n_dst;
@@ -436,8 +560,11 @@ __device__ __forceinline__ void gms_rows_body(
   constexpr int TR = kWaves * WR;                         // rows per workgroup tile
   int4v *a_lds = lds + 2 * WCH + wave * (WR * C);
   int *idx_all = reinterpret_cast<int *>(lds + 2 * WCH + kWaves * (WR * C));
-  int *gidx = idx_all + wave * 2 * WR;
-  int *didx = gidx + WR;
+  // per wave: the rows to gather -- byte offsets, two sets (this offset's and the next one's), or
+  // plain indices (!kBuf, one set) -- and the destination rows
+  unsigned *goff = reinterpret_cast<unsigned *>(idx_all + wave * 3 * WR);
+  const int *gidx = idx_all + wave * 3 * WR;
+  int *didx = idx_all + wave * 3 * WR + 2 * WR;
   const int nt0 = block_y * NT;
   const int4v *packed4 = reinterpret_cast<const int4v *>(packed);
   const size_t packed_per_k = (size_t)c_src * c_dst / E;  // chunks
@@ -462,7 +589,11 @@ __device__ __forceinline__ void gms_rows_body(
   if (owns_row) didx[lane] = in_range ? (perm ? perm[my_row] : my_row) : -1;   // my_row is a position in the plan's row order
 
   // which offsets touch this wave's rows / this workgroup's rows (from the plan)
-  const unsigned long long wave_mask = row0 < n_dst ? block_masks[row0 / 64] : 0ull;
+  unsigned long long wave_mask = row0 < n_dst ? block_masks[row0 / 64] : 0ull;
+  // (one value for the whole wave: in scalar registers where vector registers are short)
+  if constexpr (sizeof(T) == 2 || RAW == 3 || RAW == 4)
+    wave_mask = (unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(wave_mask & 0xffffffffu)) |
+              ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(wave_mask >> 32)) << 32);
   if (threadIdx.x == 0) wg_mask = 0;
   __syncthreads();
   if (lane == 0 && wave_mask) atomicOr(&wg_mask, wave_mask);
@@ -507,33 +638,54 @@ __device__ __forceinline__ void gms_rows_body(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
 
-  // weights of stage (k, slab): chunks [(slab*S + s) * nts + nt0 + nt] * 64 + lane
+  // Weights of stage (k, slab), 16-byte chunk e = threadIdx.x + kThreads * i of the stage's tile,
+  // through a buffer resource over the weight tensor: the part of a chunk's address that depends
+  // on the thread is a per-lane constant (wvoff), the part that depends on the stage is scalar.
+  //   RAW = 1: row e / (NT*4) of the slab's 2*S*8 rows of W[k], 16-byte piece e % (NT*4) of the
+  //            NT*32 columns from nt0*32 on
+  //   RAW = 2, 4: row e / C of the NT*32 rows of W[k] from nt0*32 on (c_dst rows of c_src
+  //            elements here), 16-byte piece e % C of the slab
+  //   RAW = 3: k-step e / (NT*128) of the stage, then [nt][hi, lo][lane]
+  //   RAW = 0: chunks [(slab*S + s) * nts + nt0 + nt] * 64 + lane of the re-laid copy
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      rows_resource(packed, (unsigned)k_vol * (unsigned)c_src * (unsigned)c_dst * (unsigned)sizeof(T));
+  unsigned wvoff[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    const int e = threadIdx.x + kThreads * i;
+    if constexpr (RAW == 1) wvoff[i] = (unsigned)(((e / (NT * 4)) * c_dst + (e % (NT * 4)) * E) * (int)sizeof(T));
+    else if constexpr (RAW == 2 || RAW == 4) wvoff[i] = (unsigned)(((e / C) * c_src + (e % C) * E) * (int)sizeof(T));
+    else if constexpr (RAW == 3) wvoff[i] = (unsigned)(((e / (NT * 128)) * nts * 128 + e % (NT * 128)) * 16);
+    else wvoff[i] = (unsigned)(((e / (NT * 64)) * nts * 64 + e % (NT * 64)) * 16);
+  }
   auto weights_issue = [&](int4v (&wreg)[NW], int k, int slab) {
+    if constexpr (!kBuf) {
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        const int e = threadIdx.x + kThreads * i;
+        if (NW * kThreads == WCH || e < WCH) {
+          if constexpr (RAW == 2) {
+            const int row = e / C, c = e % C;
+            wreg[i] = *reinterpret_cast<const int4v *>(
+                packed + ((size_t)k * c_dst + nt0 * 32 + row) * c_src + (size_t)(slab * C + c) * E);
+          } else {
+            const int q = e / (NT * 64), rem = e % (NT * 64);
+            wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
+          }
+        }
+      }
+      return;
+    }
+    unsigned soff;                                       // (wave-uniform: goes to the scalar offset)
+    if constexpr (RAW == 1) soff = (unsigned)(((k * c_src + slab * (C * E)) * c_dst + nt0 * 32) * (int)sizeof(T));
+    else if constexpr (RAW == 2 || RAW == 4) soff = (unsigned)(((k * c_dst + nt0 * 32) * c_src + slab * (C * E)) * (int)sizeof(T));
+    else if constexpr (RAW == 3) soff = (unsigned)(((int)packed_per_k * k + ((slab * 2) * nts + nt0) * 128) * 16);
+    else soff = (unsigned)(((int)packed_per_k * k + ((slab * S) * nts + nt0) * 64) * 16);
 #pragma unroll
     for (int i = 0; i < NW; ++i) {
       const int e = threadIdx.x + kThreads * i;
-      if (NW * kThreads == WCH || e < WCH) {
-        if constexpr (RAW == 1) {
-          // chunk e of the tile as it lies in memory: row e / (NT*4) of the slab's 2*S*8
-          // rows of W[k], 16-byte piece e % (NT*4) of the NT*32 columns from nt0*32 on
-          const int row = e / (NT * 4), c = e % (NT * 4);
-          wreg[i] = *reinterpret_cast<const int4v *>(
-              packed + ((size_t)k * c_src + slab * (C * E) + row) * c_dst + nt0 * 32 + c * E);
-        } else if constexpr (RAW == 2 || RAW == 4) {
-          // row e / C of the NT*32 rows of W[k] from nt0*32 on (c_dst rows of c_src
-          // elements here), 16-byte piece e % C of the slab
-          const int row = e / C, c = e % C;
-          wreg[i] = *reinterpret_cast<const int4v *>(
-              packed + ((size_t)k * c_dst + nt0 * 32 + row) * c_src + (size_t)(slab * C + c) * E);
-        } else if constexpr (RAW == 3) {
-          // k-step e / (NT*128) of the stage, then [nt][hi, lo][lane]
-          const int q = e / (NT * 128), rem = e % (NT * 128);
-          wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * 2 + q) * nts + nt0) * 128 + rem];
-        } else {
-          const int q = e / (NT * 64), rem = e % (NT * 64);
-          wreg[i] = packed4[packed_per_k * k + ((size_t)(slab * S + q) * nts + nt0) * 64 + rem];
-        }
-      }
+      if (NW * kThreads == WCH || e < WCH)
+        wreg[i] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wvoff[i], soff, 0));
     }
   };
   auto weights_commit = [&](const int4v (&wreg)[NW], int buf) {
@@ -564,88 +716,167 @@ __device__ __forceinline__ void gms_rows_body(
   int4v wreg[NW];
   constexpr int NV = MT * S;                              // row chunks per lane and stage
   int4v v[NV];
-  int gsel[NV];
+  int gsel[kBuf ? 1 : NV];
+  auto rows_issue = [&](int slab_, int slot_ = 0) {
+    if constexpr (kBuf) gather_issue_buf<S>(v, goff + slot_ * WR, rsrc, slab_, lane);
+    else gather_issue<T, S>(v, gsel, gidx, src, c_src, slab_, lane);
+  };
+  auto rows_commit = [&]() {
+    if constexpr (RAW == 3 || RAW == 4) gather_commit_bf3_buf(a_lds, v, lane);
+    else if constexpr (kBuf) gather_commit_buf<S>(a_lds, v, lane);
+    else gather_commit<S>(a_lds, v, gsel, lane);
+  };
 
   // prologue: stage 0 goes straight to LDS
-  if (owns_row) gidx[lane] = k_first >= 0 ? g_first : (in_range ? nbr[(size_t)k * nbr_stride + my_row] : -1);
+  if (owns_row) goff[lane] = row_offset(k_first >= 0 ? g_first : (in_range ? nbr[(size_t)k * nbr_stride + my_row] : -1));
   int g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * nbr_stride + my_row] : -1;
   wave_lds_fence();
   weights_issue(wreg, k, 0);
-  if (active) gather_issue<T, S>(v, gsel, gidx, src, c_src, 0, lane);
+  if (active) rows_issue(0);
   weights_commit(wreg, 0);
-  if (active) { if constexpr (RAW == 3 || RAW == 4) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
+  if (active) rows_commit();
   __syncthreads();
 
   int buf = 0;
-  while (true) {
-    int nk = k, nslab = slab + 1;
-    if (nslab == slabs) { nk = k_nxt; nslab = 0; }
-    const bool has_next = nk >= 0;
-    const bool next_active = has_next && ((wave_mask >> nk) & 1);
-    if (has_next) {
-      if (nk != k) {          // the row loads that used the old indices were issued a stage ago
-        if (owns_row) gidx[lane] = g_nxt;
-        wave_lds_fence();
-      }
+  if constexpr (kBuf) {
+    // Every stage is the same straight run of instructions for every wave: a wave whose rows do
+    // not use the next offset still issues its row loads (all its offsets are kAbsentRow, so
+    // they fetch nothing and return zeros) and writes the zeros to its tile, and only skips the
+    // MFMAs.  With no branch around the loads and their consumers the compiler knows exactly
+    // which loads are in flight at every point and waits for none it does not need; in
+    // particular the index load below stays in flight across the stage.
+    const int safe_row = min(my_row, n_dst - 1);
+    auto mma_stage = [&]() {
+      if constexpr (RAW == 1) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+      else if constexpr (RAW == 2) mma_slab_rawt<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+      else if constexpr (RAW == 3) mma_slab_bf3<NT>(acc, a_lds, w_lds + buf * WCH, lane);
+      else if constexpr (RAW == 4) mma_slab_bf3t<NT>(acc, a_lds, w_lds + buf * WCH, lane);
+      else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+    };
+    // Offsets are numbered in the order the tile walks them; offset j gathers through the index
+    // set j & 1.  While stage (offset j, last slab) runs, set (j + 1) & 1 serves the loads of
+    // offset j + 1 and set j & 1, which nothing reads any more, receives the offsets of offset
+    // j + 2, whose indices were requested a whole stage earlier; the indices of offset j + 3 are
+    // requested then.  So no stage starts by waiting for an index or for its way through LDS.
+    int k1 = k_nxt;                                          // the next offset (-1: none)
+    int k2 = todo ? __builtin_ctzll(todo) : -1;              // the one after
+    if (todo) todo &= todo - 1;
+    if (k1 >= 0) {                                           // (requested in the prologue, long landed)
+      const bool a1 = (wave_mask >> k1) & 1;
+      if (owns_row) goff[WR + lane] = row_offset(in_range && a1 ? g_nxt : -1);
+      wave_lds_fence();
     }
-    if (kInterleave && has_next && active && next_active) {
-      // The common stage: this stage's MFMAs with the next stage's loads between them,
-      // one row load after each (k-step, row tile) group.  A load instruction waits at
-      // issue while the CU's memory queue is full; issued in a block before the MFMAs
-      // those waits come on top of the MFMA time, issued between them they pass while
-      // the matrix pipe works off what it has.  (MFMAs and loads stay on their side of
-      // each scheduling barrier, LDS reads and address arithmetic may cross.)
-      const int4v *wl = w_lds + buf * WCH;
-      const int h = lane / 32, r = lane % 32;
+    // (nothing of the prologue is in flight any more; said explicitly, because the compiler
+    // cannot tell from the prologue's branches and would wait for loads that never were issued)
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
+    if (k2 >= 0) g_nxt = nbr[(size_t)k2 * nbr_stride + safe_row];
+    int slot = 0;
+    // One pass of the loop per stage that has a successor: request the successor's weights and
+    // rows, multiply this stage, move the successor to LDS; the last stage's products follow
+    // the loop.  (One exit test, at the top: issue and commit always run together.)
+    int nk = k, nslab = 1;
+    if (nslab == slabs) { nk = k1; nslab = 0; }
+    while (nk >= 0) {
+      const bool adv = nk != k;
+      const int nslot = adv ? slot ^ 1 : slot;
       weights_issue(wreg, nk, nslab);
-#pragma unroll
-      for (int s = 0; s < S; ++s) {
-        int4v b[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          if constexpr (RAW == 1) b[nt] = raw_weight_frag<NT, S>(wl, s, nt, lane);
-          else if constexpr (RAW == 2) b[nt] = wl[a_slot<S>(nt * 32 + r, h * S + s)];
-          else b[nt] = wl[(s * NT + nt) * 64 + lane];
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
-          const int it = s * MT + mt;                      // one of the MT * S row loads
-          gsel[it] = gidx[(it * 64 + lane) / C];
-          v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(gsel[it], 0) * c_src +
-                                                   (size_t)(nslab * C + (it * 64 + lane) % C) * E);
-          __builtin_amdgcn_sched_barrier(0x386);
-        }
+      rows_issue(nslab, nslot);
+      int k3 = -1;
+      if (adv) {
+        // (a wave that does not use an offset: all absent, also over the pair view, whose list
+        // names a row whatever the offset)
+        const bool a2 = k2 >= 0 && ((wave_mask >> k2) & 1);
+        if (owns_row) goff[slot * WR + lane] = row_offset(in_range && a2 ? g_nxt : -1);
+        wave_lds_fence();
+        k3 = todo ? __builtin_ctzll(todo) : -1;
+        if (todo) todo &= todo - 1;
+        if (k3 >= 0) g_nxt = nbr[(size_t)k3 * nbr_stride + safe_row];
       }
-    } else {
+      if (active) mma_stage();
+      wave_lds_fence();
+      rows_commit();
+      weights_commit(wreg, buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
+      active = (wave_mask >> nk) & 1;
+      k = nk;
+      slot = nslot;
+      if (adv) { k1 = k2; k2 = k3; }
+      nslab += 1;
+      if (nslab == slabs) { nk = k1; nslab = 0; }
+    }
+    if (active) mma_stage();
+  } else {
+    while (true) {
+      int nk = k, nslab = slab + 1;
+      if (nslab == slabs) { nk = k_nxt; nslab = 0; }
+      const bool has_next = nk >= 0;
+      const bool next_active = has_next && ((wave_mask >> nk) & 1);
       if (has_next) {
+        if (nk != k) {          // the row loads that used the old indices were issued a stage ago
+          if (owns_row) goff[lane] = row_offset(g_nxt);
+          wave_lds_fence();
+        }
+      }
+      if (kInterleave && has_next && active && next_active) {
+        // The common stage: this stage's MFMAs with the next stage's loads between them,
+        // one row load after each (k-step, row tile) group.  A load instruction waits at
+        // issue while the CU's memory queue is full; issued in a block before the MFMAs
+        // those waits come on top of the MFMA time, issued between them they pass while
+        // the matrix pipe works off what it has.  (MFMAs and loads stay on their side of
+        // each scheduling barrier, LDS reads and address arithmetic may cross.)
+        const int4v *wl = w_lds + buf * WCH;
+        const int h = lane / 32, r = lane % 32;
         weights_issue(wreg, nk, nslab);
-        if (next_active) gather_issue<T, S>(v, gsel, gidx, src, c_src, nslab, lane);
+  #pragma unroll
+        for (int s = 0; s < S; ++s) {
+          int4v b[NT];
+  #pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            if constexpr (RAW == 1) b[nt] = raw_weight_frag<NT, S>(wl, s, nt, lane);
+            else if constexpr (RAW == 2) b[nt] = wl[a_slot<S>(nt * 32 + r, h * S + s)];
+            else b[nt] = wl[(s * NT + nt) * 64 + lane];
+          }
+  #pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const int4v a = a_lds[a_slot<S>(mt * 32 + r, h * S + s)];
+  #pragma unroll
+            for (int nt = 0; nt < NT; ++nt) mma<T>(acc[mt][nt], a, b[nt]);
+            const int it = s * MT + mt;                      // one of the MT * S row loads
+            gsel[it] = gidx[(it * 64 + lane) / C];
+            v[it] = *reinterpret_cast<const int4v *>(src + (size_t)max(gsel[it], 0) * c_src +
+                                                     (size_t)(nslab * C + (it * 64 + lane) % C) * E);
+            __builtin_amdgcn_sched_barrier(0x386);
+          }
+        }
+      } else {
+        if (has_next) {
+          weights_issue(wreg, nk, nslab);
+          if (next_active) rows_issue(nslab);
+        }
+        if (active) {
+          if constexpr (RAW == 1) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+          else if constexpr (RAW == 2) mma_slab_rawt<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
+          else if constexpr (RAW == 3) mma_slab_bf3<NT>(acc, a_lds, w_lds + buf * WCH, lane);
+          else if constexpr (RAW == 4) mma_slab_bf3t<NT>(acc, a_lds, w_lds + buf * WCH, lane);
+          else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+        }
       }
-      if (active) {
-        if constexpr (RAW == 1) mma_slab_raw<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
-        else if constexpr (RAW == 2) mma_slab_rawt<T, NT, S>(acc, a_lds, w_lds + buf * WCH, lane);
-        else if constexpr (RAW == 3) mma_slab_bf3<NT>(acc, a_lds, w_lds + buf * WCH, lane);
-        else if constexpr (RAW == 4) mma_slab_bf3t<NT>(acc, a_lds, w_lds + buf * WCH, lane);
-        else mma_slab<T, NT, S>(acc, a_lds, w_lds + buf * WCH, 0, lane);
+      if (!has_next) break;
+      wave_lds_fence();
+      if (next_active) rows_commit();
+      weights_commit(wreg, buf ^ 1);
+      if (nk != k) {
+        k_nxt = todo ? __builtin_ctzll(todo) : -1;
+        if (todo) todo &= todo - 1;
+        g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * nbr_stride + my_row] : -1;
       }
+      __syncthreads();
+      buf ^= 1;
+      k = nk;
+      slab = nslab;
+      active = next_active;
     }
-    if (!has_next) break;
-    wave_lds_fence();
-    if (next_active) { if constexpr (RAW == 3 || RAW == 4) gather_commit_bf3(a_lds, v, gsel, lane); else gather_commit<S>(a_lds, v, gsel, lane); }
-    weights_commit(wreg, buf ^ 1);
-    if (nk != k) {
-      k_nxt = todo ? __builtin_ctzll(todo) : -1;
-      if (todo) todo &= todo - 1;
-      g_nxt = (k_nxt >= 0 && in_range) ? nbr[(size_t)k_nxt * nbr_stride + my_row] : -1;
-    }
-    __syncthreads();
-    buf ^= 1;
-    k = nk;
-    slab = nslab;
-    active = next_active;
   }
   if (wave_mask) {
     wave_lds_fence();
@@ -661,7 +892,7 @@ __global__ __launch_bounds__(kThreads, MT == 1 ? 4 : (NT == 4 ? 2 : 3)) void gms
     const T *__restrict__ src, const T *__restrict__ packed, T *__restrict__ dst,
     const int32_t *__restrict__ nbr, const unsigned long long *__restrict__ block_masks,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_dst, int k_vol,
-    int c_src, int c_dst, int part_stages, SideJob side, int pair_view) {
+    int c_src, int c_dst, int part_stages, SideJob side, int pair_view, unsigned src_bytes) {
   // the leading workgroups of the grid run the side job, if there is one
   int block_x = blockIdx.x;
   if (side.blocks) {
@@ -672,7 +903,7 @@ __global__ __launch_bounds__(kThreads, MT == 1 ? 4 : (NT == 4 ? 2 : 3)) void gms
     block_x -= side.blocks;
   }
   gms_rows_body<T, NT, S, RAW, MT>(src, packed, dst, nbr, block_masks, perm, tile_order, n_dst, k_vol, c_src,
-                                   c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z, pair_view);
+                                   c_dst, part_stages, block_x, blockIdx.y, blockIdx.z, gridDim.z, src_bytes, pair_view);
 }
 
 // ---------------------------------------------------------------------------
@@ -697,7 +928,7 @@ Shape shape_of(const GmsArgs &a) {
   // rows are read with 16-byte loads and fp16 results written as 4-byte pairs
   if (reinterpret_cast<uintptr_t>(a.src) % 16 || reinterpret_cast<uintptr_t>(a.dst) % 4) return s;
   const size_t tiles = (size_t)kWaves * kWaveRows * 2 * s.S * 16  // staging tiles
-                       + (size_t)kWaves * 2 * kWaveRows * sizeof(int);
+                       + (size_t)kWaves * 3 * kWaveRows * sizeof(int);
   s.lds_bytes = (size_t)s.c_src * s.NT * 32 * esz + tiles;      // + weights of one offset
   // wide fp16 layers: 128 columns per wave, so that a row is gathered once per 128
   // (not 64) output channels.  Costs 128 accumulator registers (2 waves per SIMD)
@@ -875,7 +1106,7 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
                                 NT == 4 ? 2 : 3, a.transpose_w);
   const bool half_tiles = rg.half_tiles;
   if (rg.drop_table) tile_order = nullptr;
-  const size_t lds_rows = half_tiles ? s.lds_rows_bytes - (size_t)kWaves * 32 * (2 * S * 16 + 2 * sizeof(int))
+  const size_t lds_rows = half_tiles ? s.lds_rows_bytes - (size_t)kWaves * 32 * (2 * S * 16 + 3 * sizeof(int))
                                      : s.lds_rows_bytes;
   const unsigned gx = rg.gx;
   if (gx == 0) return a.side.kind ? launch_side_job(a.side, a.stream) : FGMS_OK;
@@ -901,7 +1132,8 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
                       a.stream);
     kern<<<dim3(gx + (unsigned)a.side.blocks, gy, gz), kThreads, lds_rows, a.stream>>>(
         (const T *)a.src, packed, (T *)a.dst, nbr, masks, perm, tile_order, (int)a.n_dst, a.k_vol,
-        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side, pair_view ? 1 : 0);
+        s.c_src, s.c_dst, part_stages > 0 ? part_stages : 1, a.side, pair_view ? 1 : 0,
+        (unsigned)((size_t)a.n_src * s.c_src * sizeof(T)));
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -927,14 +1159,15 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
     const int32_t *__restrict__ perm, const int32_t *__restrict__ tile_order, int n_in, int k_vol,
     int c_in, int c_out, int part_stages, const T *__restrict__ in, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, SliceMap smap, int row_x, int row_y, int row_z, int wgrad_x) {
+    const int32_t *__restrict__ omap, SliceMap smap, int row_x, int row_y, int row_z, int wgrad_x,
+    unsigned gout_bytes) {
   // grid: row_x * row_y * row_z workgroups of the input gradient (tiles, column tiles,
   // parts of a tile), then wgrad_x * (tiles of dW[k]) of the weight gradient
   const int rows_total = row_x * row_y * row_z;
   if ((int)blockIdx.x < rows_total) {
     const int bx = blockIdx.x % row_x, rest = blockIdx.x / row_x;
     gms_rows_body<T, NT, S, RAWD, MT>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
-                                      part_stages, bx, rest % row_y, rest / row_y, row_z);
+                                      part_stages, bx, rest % row_y, rest / row_y, row_z, gout_bytes);
   } else {
     const int j = blockIdx.x - rows_total;
     if constexpr (BI <= 2 && BJ <= 2)
@@ -981,7 +1214,8 @@ int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArg
     kern<<<row_x * row_y * row_z + (unsigned)(g.tiles * g.ty), kThreads, lds, d.stream>>>(
         (const T *)d.src, (const T *)d.w, (T *)d.dst, p->nbr_in, p->mask_in, p->perm_in, p->tile_in,
         (int)d.n_dst, d.k_vol, d.c_in, d.c_out, part_stages, (const T *)w.in, acc32, w.kpos, w.imap, w.omap,
-        g.smap, (int)row_x, (int)row_y, (int)row_z, (int)g.tiles);
+        g.smap, (int)row_x, (int)row_y, (int)row_z, (int)g.tiles,
+        (unsigned)((size_t)d.n_src * s.c_src * sizeof(T)));
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -1136,6 +1370,13 @@ int launch_mfma_gms(const GmsArgs &a) {
   });
 }
 
+// The output-stationary kernel gathers through a buffer resource: 32-bit byte offsets, and
+// offsets at or above 2^31 stand for "no row" (gather_issue_buf).
+static bool rows_fit_buffer(const GmsArgs &a) {
+  const size_t c_src = a.transpose_w ? a.c_out : a.c_in;
+  return (size_t)a.n_src * c_src * (a.dtype == FGMS_F16 ? 2 : 4) <= kMaxBufferBytes;
+}
+
 bool planned_gms_supported(const GmsArgs &a, const Plan *p) {
   if (!p || a.dense_k >= 0 || a.k_vol > 64 || a.k_vol != p->k_vol) return false;
   if (a.transpose_w) {
@@ -1145,6 +1386,7 @@ bool planned_gms_supported(const GmsArgs &a, const Plan *p) {
   }
   // result rows are updated with 8- and 16-byte accesses
   if (reinterpret_cast<uintptr_t>(a.dst) % 16) return false;
+  if (!rows_fit_buffer(a)) return false;
   return shape_of(a).ok;
 }
 
@@ -1172,7 +1414,7 @@ bool pair_view_gms_supported(const GmsArgs &a, const Plan *p) {
   if (!p || !p->pv_in || a.dense_k >= 0 || a.k_vol != p->k_vol) return false;
   if (a.transpose_w ? (a.n_dst != p->n_in || a.n_src != p->n_out) : (a.n_dst != p->n_out || a.n_src != p->n_in))
     return false;
-  if (reinterpret_cast<uintptr_t>(a.dst) % 16) return false;
+  if (reinterpret_cast<uintptr_t>(a.dst) % 16 || !rows_fit_buffer(a)) return false;
   return shape_of(a).ok;
 }
 

@@ -32,7 +32,7 @@ __global__ void fill_i32_kernel(int32_t *__restrict__ p, size_t n, int32_t v) {
 // an output row; flags[2]: two pairs of one offset share an input row;
 // flags[3]: inside some offset the pairs are not ordered by output row;
 // flags[4], flags[5]: (64-position block, offset) combinations in use, output / input side;
-// flags[6..9]: the LDS-neighbourhood tables' (fgms_halo.hip); flags[10], flags[11]: offset bits
+// flags[6..9]: unused; flags[10], flags[11]: offset bits
 // set over all row masks of the output / input side; flags[12]: pairs in the map.  Two pairs of
 // one offset that share a row set one bit between them, so a side whose bits do not add up to
 // the pair count has such a pair (what flags[1] / flags[2] used to say).
@@ -603,8 +603,7 @@ namespace fgms {
 // order, block counts) travels to pinned host memory behind the last kernel and is read by
 // plan_resolve when the plan is first used.
 int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
-                const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
-                const int32_t *in_coords, const int32_t *out_coords, int coord_bits, void *stream,
+                const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs, void *stream,
                 bool want_bands) {
   if (!plan_out) {
     set_error("plan output pointer is null");
@@ -826,22 +825,6 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
       if (n_tiles > most_tiles) most_tiles = n_tiles;
     }
     if (most_tiles > 0) tile_order_kernel<<<2, 1024, (size_t)most_tiles * sizeof(int32_t), s>>>(ta);
-    // the tile tables of the LDS-neighbourhood kernels (plans made with coordinates only)
-    if (out_coords && in_coords) {
-      int32_t *ord[2] = {nullptr, nullptr}, *oinv[2] = {nullptr, nullptr};
-      if ((rc = halo_morton_order(out_coords, n_out, coord_bits, &ord[0], &oinv[0], &tmp, s)) == FGMS_OK) {
-        if (in_coords == out_coords && n_in == n_out) {
-          ord[1] = ord[0];
-          oinv[1] = oinv[0];
-        } else {
-          rc = halo_morton_order(in_coords, n_in, coord_bits, &ord[1], &oinv[1], &tmp, s);
-        }
-      }
-      for (int d = 0; d < 2 && rc == FGMS_OK; ++d)
-        rc = halo_build(p, d, d ? p->nbr_in : p->nbr_out, inv[d], ord[d], oinv[1 - d], ord[1 - d],
-                        p->flags + 6 + 2 * d, s);
-      if (rc != FGMS_OK) return fail(rc);
-    }
   }
   if (hipGetLastError() != hipSuccess) {
     set_error("fgms_plan_create: a build launch failed");
@@ -865,7 +848,7 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
     for (int k0 = 0; k0 < k_vol; k0 += 64) {
       fgms_plan_t *g = nullptr;
       rc = plan_create(&g, kpos + k0, in_map, out_map, n_in, n_out, k_vol - k0 < 64 ? k_vol - k0 : 64, n_pairs,
-                       in_coords, out_coords, coord_bits, stream, false);
+                       stream, false);
       if (rc != FGMS_OK) {
         fgms_plan_destroy((fgms_plan_t *)p);
         return rc;
@@ -899,7 +882,6 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       p->stages_out = b->stages_in; p->stages_in = b->stages_out;
       p->fwd_ok = b->dgrad_ok; p->dgrad_ok = b->fwd_ok;
       p->pv_in = b->pv_out; p->pv_out = b->pv_in; p->pv_mask = b->pv_mask; p->pv_rows = b->pv_rows;
-      p->halo[0] = b->halo[1]; p->halo[1] = b->halo[0];
       p->has_tables = b->has_tables;
       p->pairs_counted = b->pairs_counted;
       p->ordered = false;
@@ -932,10 +914,6 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       p->stages_out = h[4];
       p->stages_in = h[5];
       p->pairs_counted = p->has_tables ? h[12] : p->n_pairs;
-      for (int d = 0; d < 2; ++d) {
-        p->halo[d].ok = p->halo[d].order != nullptr && !h[6 + 2 * d] && !h[0];
-        p->halo[d].extra_rounds = h[7 + 2 * d];
-      }
       // The pair view, for maps sparse enough that some layer would take it (fp32 layers prefer
       // it from about 1 + 45 / channels row slots per pair on, never below 1.4): built now that
       // the counts are known, so that dense maps pay nothing.
@@ -998,19 +976,7 @@ extern "C" {
 int fgms_plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
                      const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
                      int64_t n_pairs, void *stream) {
-  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, nullptr, nullptr, 0, stream, true);
-}
-
-int fgms_plan_create_coords(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_map,
-                            const int32_t *out_map, int64_t n_in, int64_t n_out, int k_vol,
-                            int64_t n_pairs, const int32_t *in_coords, const int32_t *out_coords,
-                            int coord_bits, void *stream) {
-  if ((n_in > 0 && !in_coords) || (n_out > 0 && !out_coords) || coord_bits < 0 || coord_bits > 21) {
-    set_error("fgms_plan_create_coords: null coordinates or coord_bits outside 0..21");
-    return FGMS_E_INVALID;
-  }
-  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, in_coords, out_coords,
-                     coord_bits, stream, true);
+  return plan_create(plan_out, kpos, in_map, out_map, n_in, n_out, k_vol, n_pairs, stream, true);
 }
 
 int fgms_plan_transposed(fgms_plan_t **view_out, fgms_plan_t *base_plan) {
@@ -1062,7 +1028,6 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   }
   p->groups.clear();
   if (p->many_streams) (void)hipDeviceSynchronize();     // (blocks are handed back behind ONE stream's work)
-  halo_release(p);
   if (p->nbr_out) pool_free(p->nbr_out, p->last_stream, false);      // (nbr_in is the same block)
   if (p->mask_out) pool_free(p->mask_out, p->last_stream, false);    // (mask_in likewise)
   if (p->perm_out) pool_free(p->perm_out, p->last_stream, false);

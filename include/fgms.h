@@ -82,23 +82,6 @@ int fgms_plan_create(fgms_plan_t **plan, const int32_t *kpos,
                      int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
                      void *stream);
 /*
- * The same with the voxel coordinates of the rows (device int32 [n][3]; no counterpart in
- * the reference, whose entry points see pair lists only).  The plan additionally cuts the
- * rows, taken in Morton order of their coordinates, into spatially compact tiles of 128 and
- * lists every tile's distinct source rows (about 1.6 per destination row on surface-like
- * clouds, against 10 gathers per row); fp16 layers with 64 source channels can then run a
- * kernel that reads every distinct row once per tile into LDS and serves all offsets from
- * there (kernel policy 6; slower than the default kernel on MI355X today, kept for
- * measurement).  in_coords and out_coords may be the same pointer (submanifold maps).
- * coord_bits: every coordinate lies in [0, 2^coord_bits) (1..21; fewer bits, shorter sort),
- * or 0 for the range [-2^20, 2^20).
- */
-int fgms_plan_create_coords(fgms_plan_t **plan, const int32_t *kpos,
-                            const int32_t *in_map, const int32_t *out_map,
-                            int64_t n_in, int64_t n_out, int k_vol, int64_t n_pairs,
-                            const int32_t *in_coords, const int32_t *out_coords,
-                            int coord_bits, void *stream);
-/*
  * A plan for the same pairs with the roles of the two sides swapped (in_map and out_map
  * exchanged: the map of the transposed convolution, backend/spconv.cu:460 swaps them the
  * same way for the input gradient).  It shares the tables of `base`, which already hold both

@@ -29,8 +29,6 @@ extern "C" {
  * with atomic sums),
  * 5 = forward and input gradient over the plan's pair view whenever the plan has
  * one (plans created under this policy keep it for dense maps too),
- * 6 = forward and input gradient of fp16 layers with 64 source channels through the kernel
- * that keeps a tile's neighbourhood rows in LDS, for plans made by fgms_plan_create_coords,
  * 7 = forward and input gradient of fp16 layers with a multiple of 256 destination channels
  * through the pair-stationary kernel with 256-column workgroups even when a usable plan is
  * passed (automatic dispatch takes it where it would otherwise take the pair-stationary kernel).
