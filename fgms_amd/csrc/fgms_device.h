@@ -34,6 +34,21 @@ __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ kpos, in
   return false;
 }
 
+// Row gathers through a buffer resource: a row is addressed by a 32-bit BYTE offset into its
+// tensor (row index x row bytes), and the buffer's range check turns every load at or beyond
+// the tensor's size into zeros.  kAbsentRow is an offset no tensor reaches: a row that does not
+// exist (no neighbour through this offset, a slot past the end of a pair list) is loaded from
+// there and arrives as zeros, without a select and without touching memory.  Tensors must stay
+// below kMaxBufferBytes (checked by the host), so that kAbsentRow plus any offset inside a row
+// does not wrap round.
+constexpr unsigned kAbsentRow = 0x80000000u;
+constexpr size_t kMaxBufferBytes = 0x7fff0000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_resource(const void *base, unsigned bytes) {
+  // raw buffer: stride 0, num_records in bytes, 32-bit data format
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(__half v) { return __half2float(v); }
 

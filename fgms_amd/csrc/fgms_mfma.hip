@@ -371,20 +371,10 @@ __device__ __forceinline__ void gather_commit(int4v *__restrict__ a_lds, int4v (
   }
 }
 
-// The same two steps for the output-stationary kernel, through buffer loads: `offs` holds a
-// BYTE offset per row of the wave's tile (row index x row bytes), kAbsentRow for a row that has
-// no neighbour through this offset.  The buffer's range check turns every load at or beyond
-// `src_bytes` into zeros, so an absent row arrives as zeros by itself: no select on the way to
-// LDS, no row index kept per load, 32-bit address arithmetic.  (src_bytes < 2^31, checked by
-// the host, keeps kAbsentRow + any offset inside a row from wrapping round.)
-constexpr unsigned kAbsentRow = 0x80000000u;
-constexpr size_t kMaxBufferBytes = 0x7fff0000u;
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_resource(const void *base, unsigned bytes) {
-  // raw buffer: stride 0, num_records in bytes, 32-bit data format
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
-}
-
+// The same two steps for the output-stationary kernel, through buffer loads (see kAbsentRow):
+// `offs` holds a byte offset per row of the wave's tile, kAbsentRow for a row that has no
+// neighbour through this offset, which then arrives as zeros by itself: no select on the way
+// to LDS, no row index kept per load, 32-bit address arithmetic.
 template <int S, int N>
 __device__ __forceinline__ void gather_issue_buf(int4v (&v)[N], const unsigned *__restrict__ offs,
                                                  __amdgpu_buffer_rsrc_t rsrc, int slab, int lane) {
@@ -1160,7 +1150,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
     int c_in, int c_out, int part_stages, const T *__restrict__ in, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
     const int32_t *__restrict__ omap, SliceMap smap, int row_x, int row_y, int row_z, int wgrad_x,
-    unsigned gout_bytes) {
+    unsigned gout_bytes, unsigned in_bytes) {
   // grid: row_x * row_y * row_z workgroups of the input gradient (tiles, column tiles,
   // parts of a tile), then wgrad_x * (tiles of dW[k]) of the weight gradient
   const int rows_total = row_x * row_y * row_z;
@@ -1172,7 +1162,7 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
     const int j = blockIdx.x - rows_total;
     if constexpr (BI <= 2 && BJ <= 2)
       wgrad_wave_body<T, BI, BJ, RAWD == 4>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap,
-                                            j % wgrad_x, j / wgrad_x);
+                                            j % wgrad_x, j / wgrad_x, in_bytes, gout_bytes);
     else
       wgrad_wg_body<T, BI, BJ, RAWD == 4>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap,
                                           j % wgrad_x, j / wgrad_x);
@@ -1215,7 +1205,7 @@ int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArg
         (const T *)d.src, (const T *)d.w, (T *)d.dst, p->nbr_in, p->mask_in, p->perm_in, p->tile_in,
         (int)d.n_dst, d.k_vol, d.c_in, d.c_out, part_stages, (const T *)w.in, acc32, w.kpos, w.imap, w.omap,
         g.smap, (int)row_x, (int)row_y, (int)row_z, (int)g.tiles,
-        (unsigned)((size_t)d.n_src * s.c_src * sizeof(T)));
+        (unsigned)((size_t)d.n_src * s.c_src * sizeof(T)), (unsigned)((size_t)w.n_in * w.c_in * sizeof(T)));
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;

@@ -57,7 +57,8 @@ template <typename T, int BI, int BJ, bool SPLIT>
 __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap, SideJob side) {
+    const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, SliceMap smap, SideJob side,
+    unsigned in_bytes, unsigned gout_bytes) {
   // the leading workgroups of the grid run the side job, if there is one
   int block_x = blockIdx.x;
   if (side.blocks) {
@@ -67,7 +68,8 @@ __global__ __launch_bounds__(kThreads, 3) void wgrad_wave_kernel(
     }
     block_x -= side.blocks;
   }
-  wgrad_wave_body<T, BI, BJ, SPLIT>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, block_x, blockIdx.y);
+  wgrad_wave_body<T, BI, BJ, SPLIT>(in, gout, gw32, kpos, imap, omap, k_vol, c_in, c_out, smap, block_x, blockIdx.y,
+                                    in_bytes, gout_bytes);
 }
 
 // ---------------------------------------------------------------------------
@@ -306,7 +308,8 @@ int launch_wave(const WgradArgs &a, float *acc32) {
     ProfileScope prof(g.split ? "wgrad_wave_kernel(bf16x3)" : "wgrad_wave_kernel", a.stream);
     kern<<<dim3((unsigned)g.tiles + (unsigned)a.side.blocks, (unsigned)g.ty), kThreads, g.lds, a.stream>>>(
         (const T *)a.in, (const T *)a.gout, acc32, a.kpos, a.imap, a.omap, a.k_vol, a.c_in,
-        a.c_out, g.smap, a.side);
+        a.c_out, g.smap, a.side, (unsigned)((size_t)a.n_in * a.c_in * sizeof(T)),
+        (unsigned)((size_t)a.n_out * a.c_out * sizeof(T)));
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -372,6 +375,9 @@ bool mfma_wgrad_supported(const WgradArgs &a) {
   if (skinny_shape(a)) return true;     // (no MFMA there: the skinny kernel shares this path's accumulator)
   if (a.c_in % 32 != 0 || a.c_out % 32 != 0) return false;
   if (reinterpret_cast<uintptr_t>(a.in) % 16 || reinterpret_cast<uintptr_t>(a.gout) % 16) return false;
+  // (rows are addressed by 32-bit byte offsets through buffer resources)
+  const size_t esz = a.dtype == FGMS_F16 ? 2 : 4;
+  if ((size_t)a.n_in * a.c_in * esz > kMaxBufferBytes || (size_t)a.n_out * a.c_out * esz > kMaxBufferBytes) return false;
   return true;
 }
 

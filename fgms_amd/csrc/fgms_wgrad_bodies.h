@@ -125,9 +125,14 @@ __device__ __forceinline__ void wgrad_wave_body(
     const T *__restrict__ in, const T *__restrict__ gout, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
     const int32_t *__restrict__ omap, int k_vol, int c_in, int c_out, const SliceMap &smap,
-    int block_x, int block_y) {
+    int block_x, int block_y, unsigned in_bytes, unsigned gout_bytes) {
   using W = WT<T>;
   constexpr int E = W::E, SP = WTW<T>::stage_pairs, KP = W::step_pairs;
+  // fp16: rows through buffer loads (32-bit offsets; a slot past the end of the slice is loaded
+  // from kAbsentRow and arrives as zeros) and all of a stage's fragments requested from LDS
+  // before its first MFMA
+  constexpr bool kBufW = sizeof(T) == 2 && !SPLIT;
+  const __amdgpu_buffer_rsrc_t in_rsrc = rows_resource(in, in_bytes), gout_rsrc = rows_resource(gout, gout_bytes);
   constexpr int CI = BI * 32, CO = BJ * 32;
   constexpr int LDI = CI + W::pad, LDO = CO + W::pad;
   constexpr int NCI = CI / E, NCO = CO / E;
@@ -173,16 +178,30 @@ __device__ __forceinline__ void wgrad_wave_body(
     for (int i = 0; i < NG; ++i)
       gi[i] = omap[first + min(st * SP + (lane + 64 * i) / NCO, count - 1)];
   };
-  auto load_rows = [&]() {
+  auto load_rows = [&](int st_) {      // st_: the stage the indices in xi / gi belong to
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int cc = (lane + 64 * i) % NCI;
-      xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)xi[i] * c_in + ci0 + cc * E);
+      if constexpr (kBufW) {
+        const bool live = st_ * SP + (lane + 64 * i) / NCI < count;
+        const unsigned off = live ? (unsigned)xi[i] * (unsigned)(c_in * (int)sizeof(T)) : kAbsentRow;
+        xr[i] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(
+                                              in_rsrc, off + (unsigned)((ci0 + cc * E) * (int)sizeof(T)), 0, 0));
+      } else {
+        xr[i] = *reinterpret_cast<const int4v *>(in + (size_t)xi[i] * c_in + ci0 + cc * E);
+      }
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const int cc = (lane + 64 * i) % NCO;
-      gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
+      if constexpr (kBufW) {
+        const bool live = st_ * SP + (lane + 64 * i) / NCO < count;
+        const unsigned off = live ? (unsigned)gi[i] * (unsigned)(c_out * (int)sizeof(T)) : kAbsentRow;
+        gr[i] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(
+                                              gout_rsrc, off + (unsigned)((co0 + cc * E) * (int)sizeof(T)), 0, 0));
+      } else {
+        gr[i] = *reinterpret_cast<const int4v *>(gout + (size_t)gi[i] * c_out + co0 + cc * E);
+      }
     }
   };
   auto store_rows = [&](int st) {     // st: the stage the rows in flight belong to
@@ -191,6 +210,8 @@ __device__ __forceinline__ void wgrad_wave_body(
       const int e = lane + 64 * i;
       if constexpr (SPLIT)
         store_split_chunk(xh, xl, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count, lane);
+      else if constexpr (kBufW)
+        *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) = xr[i];
       else
         *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
             st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
@@ -200,6 +221,8 @@ __device__ __forceinline__ void wgrad_wave_body(
       const int e = lane + 64 * i;
       if constexpr (SPLIT)
         store_split_chunk(gh, gl, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count, lane);
+      else if constexpr (kBufW)
+        *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) = gr[i];
       else
         *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
             st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
@@ -212,12 +235,12 @@ __device__ __forceinline__ void wgrad_wave_body(
 
   int st = wave;
   load_idx(st);
-  load_rows();
+  load_rows(st);
   load_idx(st + 4);
   while (st < nstages) {
     store_rows(st);                 // waits for the stage's rows
     wave_fence();
-    load_rows();                    // stage st + 4, in flight during the MFMAs
+    load_rows(st + 4);              // stage st + 4, in flight during the MFMAs
     __builtin_amdgcn_sched_barrier(0);   // (rows first, then indices, both before the MFMAs:
     load_idx(st + 8);                    //  the wait for the rows then leaves the indices in flight)
     __builtin_amdgcn_sched_barrier(0);
@@ -241,6 +264,24 @@ __device__ __forceinline__ void wgrad_wave_body(
           acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ti], bl[tj], acc[ti][tj], 0, 0, 0);
           acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ti], bh[tj], acc[ti][tj], 0, 0, 0);
         }
+    } else if constexpr (kBufW) {
+      constexpr int KS = SP / KP;
+      half8 a[KS][BI], b[KS][BJ];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int ti = 0; ti < BI; ++ti) a[ks][ti] = tr_frag(x, LDI, ks * KP, ti * 32, lane);
+#pragma unroll
+        for (int tj = 0; tj < BJ; ++tj) b[ks][tj] = tr_frag(g, LDO, ks * KP, tj * 32, lane);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int ti = 0; ti < BI; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < BJ; ++tj)
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks][ti], b[ks][tj], acc[ti][tj], 0, 0, 0);
     } else {
 #pragma unroll
     for (int ks = 0; ks < SP / KP; ++ks) {
