@@ -341,7 +341,7 @@ def main():
                                  "algorithmic bytes = coordinates read + pair lists written"}
         del vox, im_, om_
     if not args.no_plan and args.surface == "cabi":
-        capi.set_kernel_policy(0 if args.policy == 6 else args.policy)
+        capi.set_kernel_policy(args.policy)
         n_np = max(5, min(50, args.steps))
         step_cabi(plan=None)
         plan_cost["no_plan_ms_per_step"] = timed(lambda: step_cabi(plan=None), n_np)
@@ -442,6 +442,12 @@ def main():
                         "unit": "TFLOP/s", "frac": ach / peak, "traffic": traffic,
                         "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
                         "mfma_flop_per_algorithmic_flop": factor,
+                        # `frac` prices the matrix pipes' work (for split bf16: three MFMA flop per
+                        # algorithmic flop); frac_algorithmic prices the useful work alone, against
+                        # the same 16-bit peak and against the fp32 MFMA peak the tensors' type has
+                        "frac_algorithmic": len(parts) * flops_pass / avg_s / 1e12 / peak,
+                        "frac_algorithmic_of_fp32_peak": (len(parts) * flops_pass / avg_s / 1e12 / PEAK_TFLOPS["f32"]
+                                                          if arith == "f32" else None),
                         "avg_kernel_ms": kernels[dom]["avg_ms"],
                         "passes_in_kernel": list(parts),
                         "algorithmic_flop": factor * len(parts) * flops_pass,

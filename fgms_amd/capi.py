@@ -14,10 +14,10 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfgms_hip.so")
 
 F32, F16 = 0, 1
 SYMBOLS = [
-    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_transposed", "fgms_plan_destroy",
+    "fgms_version", "fgms_last_error", "fgms_plan_create", "fgms_plan_check", "fgms_plan_transposed", "fgms_plan_destroy",
     "fgms_plan_usable", "fgms_plan_stats", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_wgrad_static", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
-    "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map",
+    "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map", "fgms_allocation_count",
 ]
 
 _lib = None
@@ -25,6 +25,10 @@ _lib = None
 
 class FgmsError(RuntimeError):
     pass
+
+
+class StalePlanError(FgmsError):
+    """FGMS_E_STALE: the pair lists were rewritten after the plan was made."""
 
 
 def lib():
@@ -40,6 +44,7 @@ def lib():
     L.fgms_last_error.restype = ctypes.c_char_p
     L.fgms_plan_create.argtypes = [ctypes.POINTER(vp), vp, vp, vp, i64, i64, i32, i64, vp]
     L.fgms_plan_transposed.argtypes = [ctypes.POINTER(vp), vp]
+    L.fgms_plan_check.argtypes = [vp, vp, i32]
     L.fgms_plan_destroy.argtypes = [vp]
     L.fgms_plan_destroy.restype = None
     L.fgms_plan_usable.argtypes = [vp, i32]
@@ -61,6 +66,7 @@ def lib():
     L.fgms_probe_gather.restype = i32
     L.fgms_set_kernel_policy.argtypes = [i32]
     L.fgms_set_kernel_policy.restype = None
+    L.fgms_allocation_count.restype = ctypes.c_longlong
     L.fgms_profile_enable.argtypes = [i32]
     L.fgms_profile_enable.restype = None
     L.fgms_profile_reset.restype = None
@@ -78,6 +84,8 @@ def _check(rc):
         msg = lib().fgms_last_error().decode()
         if rc == -1:
             raise ValueError(msg)
+        if rc == -4:
+            raise StalePlanError(msg)
         raise FgmsError("fgms error %d: %s" % (rc, msg))
 
 
@@ -107,6 +115,11 @@ def _need(t, name, dtype=None):
 def set_kernel_policy(policy):
     """0 automatic, 1 generic kernels only, 2 pair-stationary MFMA even with a plan."""
     lib().fgms_set_kernel_policy(int(policy))
+
+
+def allocation_count():
+    """Device / pinned allocations the library has made so far (``fgms_allocation_count``)."""
+    return int(lib().fgms_allocation_count())
 
 
 def profile_enable(on=True):
@@ -153,6 +166,12 @@ class Plan:
         view._h = ctypes.c_void_p()
         _check(lib().fgms_plan_transposed(ctypes.byref(view._h), self._h))
         return view
+
+    def check(self, with_next_launch=False):
+        """Has the pair lists checked against the fingerprint the plan was built with
+        (``fgms_plan_check``): by a small kernel queued now, or as part of the next launch that
+        reads the plan; raises StalePlanError once an earlier check has found them changed."""
+        _check(lib().fgms_plan_check(self._h, _stream(), int(with_next_launch)))
 
     def usable(self, for_dgrad=False):
         return bool(lib().fgms_plan_usable(self._h, int(for_dgrad)))
@@ -240,10 +259,11 @@ def dgrad(out_grad, kernel, in_grad, kpos, in_map, out_map, plan=None):
         in_map.numel(), _dtype(out_grad), _ph(plan), _stream()))
 
 
-def build_kernel_map(in_coords, out_coords, offsets, stride=1, skip_offset=None, capacity=None):
+def build_kernel_map(in_coords, out_coords, offsets, stride=1, skip_offset=None, capacity=None, into=None):
     """Pair lists of a kernel map from int32 voxel coordinates on the device.
     Returns (in_map, out_map, kernel_nnz, kpos): device int32 tensors, the maps trimmed
-    to the number of pairs found."""
+    to the number of pairs found.  into=(in_map, out_map, kernel_nnz, kpos): write into these
+    tensors (through their data pointers, as a native builder does) and return them untrimmed."""
     import numpy as np
     import torch
     for t, n in ((in_coords, "in_coords"), (out_coords, "out_coords")):
@@ -253,15 +273,21 @@ def build_kernel_map(in_coords, out_coords, offsets, stride=1, skip_offset=None,
     k_vol = len(offs)
     n_in, n_out = in_coords.shape[0], out_coords.shape[0]
     cap = k_vol * n_out if capacity is None else int(capacity)
-    in_map = torch.empty(max(cap, 1), dtype=torch.int32, device=in_coords.device)
-    out_map = torch.empty(max(cap, 1), dtype=torch.int32, device=in_coords.device)
-    knnz = torch.empty(k_vol, dtype=torch.int32, device=in_coords.device)
-    kpos = torch.empty(k_vol + 1, dtype=torch.int32, device=in_coords.device)
+    if into is not None:
+        in_map, out_map, knnz, kpos = into
+        cap = min(in_map.numel(), out_map.numel())
+    else:
+        in_map = torch.empty(max(cap, 1), dtype=torch.int32, device=in_coords.device)
+        out_map = torch.empty(max(cap, 1), dtype=torch.int32, device=in_coords.device)
+        knnz = torch.empty(k_vol, dtype=torch.int32, device=in_coords.device)
+        kpos = torch.empty(k_vol + 1, dtype=torch.int32, device=in_coords.device)
     found = ctypes.c_int64(0)
     _check(lib().fgms_build_kernel_map(
         _p(in_coords), n_in, _p(out_coords), n_out, offs.ctypes.data_as(ctypes.c_void_p), k_vol,
         int(stride), -1 if skip_offset is None else int(skip_offset), _p(in_map), _p(out_map), cap,
         _p(knnz), _p(kpos), ctypes.byref(found), _stream()))
+    if into is not None:
+        return in_map, out_map, knnz, kpos
     return in_map[:found.value], out_map[:found.value], knnz, kpos
 
 

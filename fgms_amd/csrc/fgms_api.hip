@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -52,6 +53,10 @@ size_t workspace_bytes(hipStream_t stream, int slot) {
   return it == g_ws.end() ? 0 : it->second.bytes;
 }
 
+// Device / pinned allocations the library has made since it was loaded (fgms_allocation_count).
+std::atomic<long long> g_allocations{0};
+void note_allocation() { g_allocations.fetch_add(1, std::memory_order_relaxed); }
+
 int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *fresh) {
   if (fresh) *fresh = false;
   int dev = 0;
@@ -74,6 +79,7 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *
       b.bytes = 0;
     }
     size_t want = bytes + bytes / 4 + 4096;
+    note_allocation();
     if (hipMalloc(&b.ptr, want) != hipSuccess) {
       b.ptr = nullptr;
       set_error("workspace allocation of %zu bytes failed", want);
@@ -159,6 +165,7 @@ int pool_alloc(void **ptr, size_t bytes, hipStream_t user) {
     return FGMS_OK;
   }
   void *q = nullptr;
+  note_allocation();
   if (hipMalloc(&q, bytes) != hipSuccess) {
     // give cached blocks back to the driver and try once more
     pool_trim(0);
@@ -384,6 +391,16 @@ int check_mid(int separate_mid, int64_t n_in, int64_t n_out) {
 
 using namespace fgms;
 
+// A fingerprint check of the plan that none of the call's launches carried as a side job goes
+// out as a launch of its own when the entry point returns.
+namespace {
+struct CheckFlush {
+  const Plan *p;
+  hipStream_t s;
+  ~CheckFlush() { if (p) (void)plan_flush_check(p, s); }
+};
+}  // namespace
+
 extern "C" {
 
 const char *fgms_version(void) { return "fgms-hip 0.1 (gfx950)"; }
@@ -391,6 +408,7 @@ const char *fgms_last_error(void) { return g_error; }
 void fgms_set_kernel_policy(int policy) { g_policy = policy; }
 
 void fgms_profile_enable(int on) { g_prof_on = on != 0; }
+long long fgms_allocation_count(void) { return g_allocations.load(std::memory_order_relaxed); }
 
 void fgms_profile_reset(void) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
@@ -439,6 +457,7 @@ int fgms_fusion_fwd(const void *in_feats, const void *kernel, int sum_nnz, void 
     if ((rc = run_gms(d, nullptr))) return rc;
   }
   const Plan *p = plan_resolve(plan, s, &rc);
+  CheckFlush flush{p, s};
   if (rc) return rc;
   return run_gms(a, p);
 }
@@ -477,6 +496,7 @@ int fgms_fwd(const void *in_feats, const void *kernel, int sum_nnz, void *out_fe
                        c_in, c_out, k_vol, total, dtype, s);
   a.reduced = arch80 != 0 && dtype == FGMS_F32;
   const Plan *p = plan_resolve(plan, s, &rc);
+  CheckFlush flush{p, s};
   if (rc) return rc;
   if ((rc = run_gms(a, p))) return rc;
   if (separate_mid) {
@@ -503,6 +523,7 @@ int fgms_dgrad(const void *out_feats_grad, const void *kernel, void *in_feats_gr
   a.n_pairs = n_pairs; a.transpose_w = true; a.dense_k = -1; a.n_dense = 0; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
   const Plan *p = plan_resolve(plan, a.stream, &rc);
+  CheckFlush flush{p, a.stream};
   if (rc) return rc;
   return run_gms(a, p);
 }
@@ -520,6 +541,7 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
   a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
   a.plan = plan_resolve(plan, a.stream, &rc);
+  CheckFlush flush{a.plan, a.stream};
   if (rc) return rc;
   return run_wgrad(a);
 }
@@ -536,8 +558,9 @@ int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *ke
   a.imap = in_map; a.omap = out_map; a.n_in = n_in; a.n_out = n_out; a.c_in = c_in;
   a.c_out = c_out; a.k_vol = k_vol; a.n_pairs = n_pairs; a.dtype = dtype;
   a.stream = (hipStream_t)stream;
-  a.plan = plan_resolve(plan, a.stream, &rc);
-  if (rc) return rc;
+  // (resolving a plan on its first use waits for the build and may allocate the pair view: this
+  // entry point does neither, it takes the plan's row bands only if they are known already)
+  a.plan = plan_if_resolved(plan);
   return wgrad_static(a);
 }
 
@@ -554,6 +577,7 @@ int fgms_bwd(const void *out_feats_grad, const void *in_feats, const void *kerne
                          c_in, c_out, k_vol, n_pairs, dtype)))
     return rc;
   const Plan *p = plan_resolve(plan, (hipStream_t)stream, &rc);
+  CheckFlush flush{p, (hipStream_t)stream};
   if (rc) return rc;
   GmsArgs d{};
   d.src = out_feats_grad; d.w = kernel; d.dst = in_feats_grad; d.kpos = kpos;

@@ -119,6 +119,63 @@ __device__ __forceinline__ void add_and_clear_elements(__half *__restrict__ dst,
   }
 }
 
+// Fingerprint of the pair lists: the sum, over a fixed sample of positions (every `stride`-th
+// pair) and over kpos, of a hash of (position, values).  Taken by the build (inside
+// pair_masks_kernel) and again by fgms_plan_check; sums of 64-bit hashes, so the order in which
+// threads add does not matter.
+__device__ __forceinline__ unsigned long long print_hash(unsigned long long a, unsigned b, unsigned c) {
+  unsigned long long x = a * 0x9E3779B97F4A7C15ull + ((unsigned long long)b << 32 | c);
+  x ^= x >> 31; x *= 0xBF58476D1CE4E5B9ull; x ^= x >> 29;
+  return x;
+}
+constexpr int kPrintSamples = 4096;
+__host__ __device__ inline int print_stride(int n_pairs) { return n_pairs > kPrintSamples ? n_pairs / kPrintSamples : 1; }
+
+// This thread's share of the fingerprint: pair j if it is a sampled one, and entry j - first of
+// kpos for the first k_vol + 1 pairs.  (first = kpos[0], total = pairs in the lists.)
+__device__ __forceinline__ unsigned long long print_share(const int32_t *__restrict__ kpos,
+                                                          const int32_t *__restrict__ imap,
+                                                          const int32_t *__restrict__ omap, int k_vol,
+                                                          int first, int total, int j) {
+  unsigned long long v = 0;
+  const int rel = j - first, stride = print_stride(total - first);
+  if (rel % stride == 0) v += print_hash((unsigned long long)rel, (unsigned)imap[j], (unsigned)omap[j]);
+  if (rel <= k_vol) v += print_hash(0x100000000ull + rel, (unsigned)kpos[rel], 0u);
+  return v;
+}
+
+
+// The fingerprint taken again from the lists as they are now, by one workgroup (the sample is
+// 4 096 pairs), and compared with the build's; a difference raises the sticky flag, in device
+// memory and in the plan's pinned block (fgms_plan_check).
+__device__ __forceinline__ void plan_check_block(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+                                                 const int32_t *__restrict__ omap, int k_vol, int n_pairs,
+                                                 int *__restrict__ flags, int *__restrict__ host) {
+  __shared__ unsigned long long part[16];
+  const int threads = blockDim.x;
+  const int first = kpos[0], total = min(kpos[k_vol], n_pairs);
+  const int stride = print_stride(total - first);
+  unsigned long long v = 0;
+  // the sampled pairs, then the pairs whose threads carried kpos in the build
+  for (int s = threadIdx.x; first + (long long)s * stride < total; s += threads) {
+    const int j = first + s * stride;
+    v += print_hash((unsigned long long)(j - first), (unsigned)imap[j], (unsigned)omap[j]);
+  }
+  for (int rel = threadIdx.x; rel <= k_vol && first + rel < total; rel += threads)
+    v += print_hash(0x100000000ull + rel, (unsigned)kpos[rel], 0u);
+  for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
+  if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long sum = 0;
+    for (int w = 0; w < threads / 64; ++w) sum += part[w];
+    if (sum != *reinterpret_cast<const unsigned long long *>(flags + kFlagPrint)) {
+      flags[kFlagStale] = 1;
+      if (host) host[kFlagStale] = 1;
+    }
+  }
+}
+
 // The side job of a launch, run by workgroup `block` of its job.blocks workgroups.
 __device__ __forceinline__ void run_side_job(const SideJob &job, int block) {
   const size_t first = (size_t)block * blockDim.x + threadIdx.x;
@@ -132,6 +189,10 @@ __device__ __forceinline__ void run_side_job(const SideJob &job, int block) {
                                   job.c_out, job.S, job.transpose != 0, first, stride);
   } else if (job.kind == 2) {
     add_and_clear_elements((__half *)job.dst, job.acc, job.n, first, stride);
+  } else if (job.kind == 3) {
+    if (block == 0)
+      plan_check_block((const int32_t *)job.src, (const int32_t *)job.dst, job.omap, job.k_vol, (int)job.n,
+                       job.flags, job.host);
   }
 }
 

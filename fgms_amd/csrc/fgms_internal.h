@@ -37,7 +37,9 @@ void set_error(const char *fmt, ...);
 //   kind 1: re-lay the weights `src` into MFMA fragment order at `dst` (what
 //           pack_weights_kernel does), for the launch that follows on the stream;
 //   kind 2: dst[i] += acc[i] rounded once to fp16 and acc[i] = 0 (what add_and_clear_kernel
-//           does) for the fp32 accumulator the previous launch on the stream filled.
+//           does) for the fp32 accumulator the previous launch on the stream filled;
+//   kind 3: the plan's fingerprint check (fgms_plan_check): src = kpos, dst = in_map, omap,
+//           n = the pair bound, k_vol; one workgroup works, the others of the job leave.
 struct SideJob {
   int kind;      // 0: none
   int blocks;
@@ -46,6 +48,8 @@ struct SideJob {
   float *acc;
   size_t n;      // elements
   int k_vol, c_in, c_out, S, transpose, dtype;
+  const int32_t *omap;
+  int *flags, *host;
 };
 
 // dense:   gmap == smap == nullptr means the identity map over n_dense rows of
@@ -96,7 +100,9 @@ struct WgradArgs {
   float *acc_override;
 };
 
-constexpr int kPlanFlags = 13;      // ints the plan build reports back (see fgms_plan.hip)
+constexpr int kPlanFlags = 16;      // ints the plan build reports back (see fgms_plan.hip)
+constexpr int kFlagStale = 13;      // flags[13]: a later check found another fingerprint (fgms_plan_check)
+constexpr int kFlagPrint = 14;      // flags[14], flags[15]: fingerprint of the pair lists (one 64-bit word)
 
 // Plan: neighbour tables built from the pair lists.
 struct Plan {
@@ -114,7 +120,11 @@ struct Plan {
   std::vector<Plan *> groups;   // k_vol > 64: one plan per 64 offsets (owned)
   bool has_tables;        // k_vol <= 64: neighbour tables and masks exist (else the plan is the weight gradient's bands only)
   const int32_t *kpos, *in_map, *out_map;    // the caller's lists (for the pair view, built on first use)
-  hipStream_t pv_stream;
+  hipStream_t pv_stream;        // the stream the pair view was built on
+  hipEvent_t pv_ready;          // fires behind its last kernel (launches on other streams wait for it)
+  hipStream_t create_stream;    // the stream the build was queued on
+  mutable bool checked;         // a fingerprint check has been queued at least once (host_flags[kFlagStale] means something)
+  mutable bool check_pending;   // fgms_plan_check was called: the next launch through the plan carries the check
   int k_vol;
   int64_t n_in, n_out, n_pairs;
   // Destination rows are visited in a plan-chosen order (rows with the same set
@@ -235,6 +245,13 @@ inline void plan_touch(const Plan *p, hipStream_t stream) {
 }
 // The plan with its build results known, or nullptr (see fgms_plan.hip).
 const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc);
+const Plan *plan_if_resolved(fgms_plan_t *plan);
+// fgms_plan_check only marks the plan; the check itself rides along with the next launch that
+// reads the plan and can carry a side job (plan_take_check fills one in and returns true), or
+// goes out as a small launch of its own behind the call (plan_flush_check).
+bool plan_take_check(const Plan *p, SideJob *job);
+int plan_flush_check(const Plan *p, hipStream_t stream);
+void note_allocation();      // counts a hipMalloc / hipHostMalloc of the library (fgms_allocation_count)
 int build_kernel_map(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
                      const int32_t *offsets_host, int k_vol, int stride, int skip_offset,
                      int32_t *in_map, int32_t *out_map, int64_t capacity, int32_t *kernel_nnz,

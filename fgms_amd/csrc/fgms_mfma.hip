@@ -1150,10 +1150,15 @@ __global__ __launch_bounds__(kThreads, NT == 4 ? 2 : 3) void bwd_fused_kernel(
     int c_in, int c_out, int part_stages, const T *__restrict__ in, float *__restrict__ gw32,
     const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
     const int32_t *__restrict__ omap, SliceMap smap, int row_x, int row_y, int row_z, int wgrad_x,
-    unsigned gout_bytes, unsigned in_bytes) {
+    unsigned gout_bytes, unsigned in_bytes, int wgrad_blocks, SideJob check) {
   // grid: row_x * row_y * row_z workgroups of the input gradient (tiles, column tiles,
-  // parts of a tile), then wgrad_x * (tiles of dW[k]) of the weight gradient
+  // parts of a tile), then wgrad_x * (tiles of dW[k]) of the weight gradient, then those of a
+  // side job (the plan's fingerprint check), if there is one
   const int rows_total = row_x * row_y * row_z;
+  if ((int)blockIdx.x >= rows_total + wgrad_blocks) {
+    run_side_job(check, (int)blockIdx.x - rows_total - wgrad_blocks);
+    return;
+  }
   if ((int)blockIdx.x < rows_total) {
     const int bx = blockIdx.x % row_x, rest = blockIdx.x / row_x;
     gms_rows_body<T, NT, S, RAWD, MT>(gout, w, gin, nbr, block_masks, perm, tile_order, n_in, k_vol, c_out, c_in,
@@ -1201,11 +1206,14 @@ int launch_fused(const GmsArgs &d, const Shape &s, const Plan *p, const WgradArg
   { const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)lds); if (rc_lds != FGMS_OK) return rc_lds; }
   {
     ProfileScope prof(split ? "bwd_fused_kernel(bf16x3)" : "bwd_fused_kernel", d.stream);
-    kern<<<row_x * row_y * row_z + (unsigned)(g.tiles * g.ty), kThreads, lds, d.stream>>>(
+    SideJob check{};
+    (void)plan_take_check(p, &check);
+    kern<<<row_x * row_y * row_z + (unsigned)(g.tiles * g.ty) + (unsigned)check.blocks, kThreads, lds, d.stream>>>(
         (const T *)d.src, (const T *)d.w, (T *)d.dst, p->nbr_in, p->mask_in, p->perm_in, p->tile_in,
         (int)d.n_dst, d.k_vol, d.c_in, d.c_out, part_stages, (const T *)w.in, acc32, w.kpos, w.imap, w.omap,
         g.smap, (int)row_x, (int)row_y, (int)row_z, (int)g.tiles,
-        (unsigned)((size_t)d.n_src * s.c_src * sizeof(T)), (unsigned)((size_t)w.n_in * w.c_in * sizeof(T)));
+        (unsigned)((size_t)d.n_src * s.c_src * sizeof(T)), (unsigned)((size_t)w.n_in * w.c_in * sizeof(T)),
+        (int)(g.tiles * g.ty), check);
   }
   FGMS_HIP_TRY(hipGetLastError());
   return FGMS_OK;
@@ -1391,12 +1399,16 @@ int launch_planned_gms(const GmsArgs &a, const Plan *p) {
   const int32_t *perm = a.transpose_w ? p->perm_in : p->perm_out;
   const int32_t *tile_order = a.transpose_w ? p->tile_in : p->tile_out;
   const int tile_grid = a.transpose_w ? p->tile_grid_in : p->tile_grid_out;
+  // (a pending fingerprint check of the plan rides along as the launch's side job)
+  GmsArgs with_check = a;
+  if (!with_check.side.kind) (void)plan_take_check(p, &with_check.side);
+  const GmsArgs &a_ = with_check;
   if (a.dtype == FGMS_F16)
     return dispatch_rows_shape<__half>(s, [&](auto nt, auto sv) {
-      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm, tile_order, tile_grid);
+      return launch_rows<__half, decltype(nt)::value, decltype(sv)::value>(a_, s, nbr, masks, perm, tile_order, tile_grid);
     });
   return dispatch_rows_shape<float>(s, [&](auto nt, auto sv) {
-    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a, s, nbr, masks, perm, tile_order, tile_grid);
+    return launch_rows<float, decltype(nt)::value, decltype(sv)::value>(a_, s, nbr, masks, perm, tile_order, tile_grid);
   });
 }
 
@@ -1413,6 +1425,8 @@ int launch_pair_view_gms(const GmsArgs &a, const Plan *p) {
     set_error("launch_pair_view_gms: unsupported shape or plan");
     return FGMS_E_INVALID;
   }
+  // (the view was built on the stream that first resolved the plan)
+  if (p->pv_ready && a.stream != p->pv_stream) FGMS_HIP_TRY(hipStreamWaitEvent(a.stream, p->pv_ready, 0));
   // the virtual rows stand in for the destination rows: tiles, the in-range test and the
   // choice of the wave tile's width go by their number
   GmsArgs v = a;

@@ -55,6 +55,10 @@ __global__ void pair_masks_kernel(const int32_t *__restrict__ kpos, const int32_
   const int k = lo;
   const int i = imap[j], o = omap[j];
   if (j == kpos[0]) flags[12] = min(total, n_pairs) - kpos[0];
+  {
+    const unsigned long long share = print_share(kpos, imap, omap, k_vol, kpos[0], min(total, n_pairs), j);
+    if (share) atomicAdd(reinterpret_cast<unsigned long long *>(flags + kFlagPrint), share);
+  }
   if (i < 0 || i >= n_in || o < 0 || o >= n_out) {
     flags[0] = 1;
     return;
@@ -562,6 +566,7 @@ int *pinned_flags_get() {
     }
   }
   int *q = nullptr;
+  note_allocation();
   if (hipHostMalloc((void **)&q, kPlanFlags * sizeof(int), hipHostMallocDefault) != hipSuccess) return nullptr;
   return q;
 }
@@ -569,6 +574,16 @@ int *pinned_flags_get() {
 void pinned_flags_put(int *q) {
   std::lock_guard<std::mutex> lock(g_pinned_mutex);
   g_pinned_free.push_back(q);
+}
+
+// fgms_plan_check: the fingerprint taken again from the lists as they are now (one workgroup:
+// the sample is 4 096 pairs), compared with the build's; a difference raises the sticky flag,
+// in device memory and in the plan's pinned block.
+__global__ __launch_bounds__(1024) void plan_check_kernel(const int32_t *__restrict__ kpos,
+                                                          const int32_t *__restrict__ imap,
+                                                          const int32_t *__restrict__ omap, int k_vol, int n_pairs,
+                                                          int *__restrict__ flags, int *__restrict__ host) {
+  plan_check_block(kpos, imap, omap, k_vol, n_pairs, flags, host);
 }
 
 // The build's findings -> pinned host memory (mapped into the device's address space).
@@ -627,10 +642,14 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   Plan *p = new Plan();          // (value-initialised: every field starts out zero)
   p->k_vol = k_vol; p->n_in = n_in; p->n_out = n_out; p->n_pairs = n_pairs;
   p->last_stream = s;
+  p->create_stream = s;
   p->kpos = kpos; p->in_map = in_map; p->out_map = out_map;
   int rc = FGMS_OK;
   std::vector<void *> tmp;          // temporaries: handed back to the pool behind the last kernel
+  hipStream_t side_in_use = nullptr;     // the library's own stream, once work of this build is queued on it
   auto fail = [&](int code) {
+    // (blocks are handed back behind `s` alone: the side stream's work must have finished)
+    if (side_in_use) (void)hipStreamSynchronize(side_in_use);
     for (void *q : tmp) pool_free(q, s, false);
     fgms_plan_destroy((fgms_plan_t *)p);
     return code;
@@ -641,7 +660,8 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
     return true;
   };
   if (hipGetDevice(&p->device) != hipSuccess) return fail(FGMS_E_HIP);
-  if (!(p->host_flags = pinned_flags_get()) ||
+  if ((p->host_flags = pinned_flags_get())) p->host_flags[kFlagStale] = 0;     // (a recycled block: the flag is read before the build has run)
+  if (!p->host_flags ||
       hipEventCreateWithFlags(&p->ready, hipEventDisableTiming) != hipSuccess) {
     set_error("fgms_plan_create: pinned flag block / event creation failed");
     return fail(FGMS_E_NOMEM);
@@ -708,6 +728,7 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   };
   {
     hipStream_t sb = s2 ? s2 : s;
+    side_in_use = s2;
     if (want_bands) {
       band_bounds_kernel<<<(unsigned)k_vol, 128, 0, sb>>>(kpos, out_map, (int)n_pairs, p->band_count,
                                                           band_rows > 0 ? band_rows : 1, p->band_start);
@@ -864,10 +885,77 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
 // known (waiting for the build if it has not finished yet), nullptr when they cannot be had
 // now (the stream is being captured into a graph: the caller then takes the kernels that need
 // no plan) or when the map turned out to be invalid (*rc = FGMS_E_INVALID).
+// The plan if its build results are already known to the host, else nullptr: never waits,
+// never allocates, never launches (for the entry point that promises that).
+const Plan *plan_if_resolved(fgms_plan_t *plan) {
+  Plan *p = (Plan *)plan;
+  if (!p) return nullptr;
+  std::lock_guard<std::mutex> lock(p->mutex);
+  return p->resolved && !p->invalid ? p : nullptr;
+}
+
+static Plan *check_owner(const Plan *p) { return const_cast<Plan *>(p->base ? p->base : p); }
+
+bool plan_take_check(const Plan *p, SideJob *job) {
+  Plan *b = check_owner(p);
+  if (!b->check_pending || !b->has_tables || !b->flags || b->n_pairs == 0) return false;
+  if (!b->resolved) return false;     // (the build may still be running: the fingerprint is not final)
+  int *host_dev = nullptr;
+  if (hipHostGetDevicePointer((void **)&host_dev, b->host_flags, 0) != hipSuccess) host_dev = nullptr;
+  *job = SideJob{};
+  job->kind = 3;
+  job->blocks = 8;                 // (a multiple of 8: the workgroups behind keep their XCDs)
+  job->src = b->kpos;
+  job->dst = const_cast<int32_t *>(b->in_map);
+  job->omap = b->out_map;
+  job->n = (size_t)b->n_pairs;
+  job->k_vol = b->k_vol;
+  job->flags = b->flags;
+  job->host = host_dev;
+  b->check_pending = false;
+  b->checked = true;
+  return true;
+}
+
+int plan_flush_check(const Plan *p, hipStream_t s) {
+  Plan *b = check_owner(p);
+  for (Plan *g : b->groups) {
+    const int rc = plan_flush_check(g, s);
+    if (rc != FGMS_OK) return rc;
+  }
+  if (!b->check_pending) return FGMS_OK;
+  b->check_pending = false;
+  if (!b->has_tables || !b->flags || b->n_pairs == 0) return FGMS_OK;
+  int *host_dev = nullptr;
+  if (hipHostGetDevicePointer((void **)&host_dev, b->host_flags, 0) != hipSuccess) host_dev = nullptr;
+  // (queued behind the build if that ran on another stream: the fingerprint must be final)
+  // (a resolved plan's build has finished; no event is queried then, which a stream under
+  // capture would not allow)
+  if (!b->resolved && s != b->create_stream) FGMS_HIP_TRY(hipStreamWaitEvent(s, b->ready, 0));
+  plan_check_kernel<<<1, 1024, 0, s>>>(b->kpos, b->in_map, b->out_map, b->k_vol, (int)b->n_pairs, b->flags, host_dev);
+  FGMS_HIP_TRY(hipGetLastError());
+  b->checked = true;
+  return FGMS_OK;
+}
+
+// Has an earlier fgms_plan_check found the lists changed?  (Reads the pinned block; no wait.)
+static bool plan_is_stale(const Plan *p) {
+  const Plan *b = p->base ? p->base : p;
+  if (b->checked && b->host_flags && b->host_flags[kFlagStale]) return true;
+  for (const Plan *g : b->groups)
+    if (g->checked && g->host_flags && g->host_flags[kFlagStale]) return true;
+  return false;
+}
+
 const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
   *rc = FGMS_OK;
   Plan *p = (Plan *)plan;
   if (!p) return nullptr;
+  if (plan_is_stale(p)) {
+    set_error("plan: the pair lists were rewritten after the plan was made (make a new plan)");
+    *rc = FGMS_E_STALE;
+    return nullptr;
+  }
   if (p->base && !p->resolved) {
     // a transposed view: the base's tables with the sides swapped
     const Plan *b = plan_resolve((fgms_plan_t *)p->base, stream, rc);
@@ -882,6 +970,7 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       p->stages_out = b->stages_in; p->stages_in = b->stages_out;
       p->fwd_ok = b->dgrad_ok; p->dgrad_ok = b->fwd_ok;
       p->pv_in = b->pv_out; p->pv_out = b->pv_in; p->pv_mask = b->pv_mask; p->pv_rows = b->pv_rows;
+      p->pv_ready = b->pv_ready; p->pv_stream = b->pv_stream;
       p->has_tables = b->has_tables;
       p->pairs_counted = b->pairs_counted;
       p->ordered = false;
@@ -921,7 +1010,10 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
       const int most = p->stages_out > p->stages_in ? p->stages_out : p->stages_in;
       if (!p->invalid && pair_view && p->has_tables && p->pairs_counted > 0 &&
           (kernel_policy() == 5 || (double)most * 64.0 >= 1.35 * (double)p->pairs_counted)) {
-        hipStream_t s = stream;
+        // (a caller that names no stream -- fgms_plan_usable, fgms_plan_stats -- must not put the
+        // view on the legacy null stream, which the streams torch makes do not wait for: the
+        // stream the plan itself was built on takes it)
+        hipStream_t s = stream ? stream : p->create_stream;
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         const bool capturing = s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
         const int64_t rows = (p->pairs_counted + 64 * (int64_t)p->k_vol + 255) / 256 * 256;
@@ -934,6 +1026,15 @@ const Plan *plan_resolve(fgms_plan_t *plan, hipStream_t stream, int *rc) {
           pair_view_kernel<<<(unsigned)((p->n_pairs + 255) / 256), 256, 0, s>>>(
               p->kpos, p->in_map, p->out_map, p->k_vol, (int)p->n_pairs, (long long)rows, p->pv_in, p->pv_out,
               p->pv_mask);
+          // launches on other streams wait for this event (launch_pair_view_gms, the destroy path)
+          if (hipGetLastError() != hipSuccess ||
+              hipEventCreateWithFlags(&p->pv_ready, hipEventDisableTiming) != hipSuccess ||
+              hipEventRecord(p->pv_ready, s) != hipSuccess) {
+            // without the event nothing else can be ordered behind the build: finish it here
+            (void)hipStreamSynchronize(s);
+            if (p->pv_ready) (void)hipEventDestroy(p->pv_ready);
+            p->pv_ready = nullptr;
+          }
           p->pv_rows = rows;
           p->pv_stream = s;
         } else {
@@ -1008,7 +1109,7 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
     bool free_base = false;
     {
       std::lock_guard<std::mutex> lock(b->mutex);
-      if (p->last_stream != b->last_stream) b->many_streams = true;
+      if (p->last_stream != b->last_stream || p->many_streams) b->many_streams = true;
       b->views -= 1;
       free_base = b->views == 0 && b->destroyed;
     }
@@ -1036,6 +1137,11 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->band_cells) pool_free(p->band_cells, p->last_stream, false);
   if (p->tile_out) pool_free(p->tile_out, p->last_stream, false);
   if (p->tile_in) pool_free(p->tile_in, p->last_stream, false);
+  if (p->pv_ready) {
+    // the view may have been built on another stream than the one the blocks are handed back behind
+    if (p->pv_stream != p->last_stream) (void)hipStreamWaitEvent(p->last_stream, p->pv_ready, 0);
+    (void)hipEventDestroy(p->pv_ready);
+  }
   if (p->pv_in) pool_free(p->pv_in, p->last_stream, false);
   if (p->pv_out) pool_free(p->pv_out, p->last_stream, false);
   if (p->pv_mask) pool_free(p->pv_mask, p->last_stream, false);
@@ -1047,6 +1153,20 @@ void fgms_plan_destroy(fgms_plan_t *plan) {
   if (p->flags) pool_free(p->flags, p->last_stream, false);
   if (p->host_flags) pinned_flags_put(p->host_flags);
   delete p;
+}
+
+int fgms_plan_check(fgms_plan_t *plan, void *stream, int with_next_launch) {
+  Plan *p = (Plan *)plan;
+  if (!p) return FGMS_OK;
+  Plan *b = p->base ? p->base : p;           // (a view shares its base's lists and flags)
+  if (plan_is_stale(p)) {
+    set_error("plan: the pair lists were rewritten after the plan was made (make a new plan)");
+    return FGMS_E_STALE;
+  }
+  b->check_pending = true;
+  for (Plan *g : b->groups) g->check_pending = true;
+  if (with_next_launch) return FGMS_OK;
+  return plan_flush_check(p, (hipStream_t)stream);
 }
 
 int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad) {

@@ -9,9 +9,10 @@
 //    triple (asynchronously: the call queues the build and goes on) and kept in a
 //    small cache; an entry holds references to the three tensors, so their storage
 //    cannot be recycled while it is cached, and is dropped when one of them is
-//    modified in place (version counter; writes through raw pointers do not bump
-//    it, and tensors made under inference mode have none: clear the cache after
-//    rewriting such a map).  A call with in_map and out_map exchanged (the
+//    modified in place (version counter).  Writes through raw pointers do not bump
+//    it, and tensors made under inference mode have none: every cache hit therefore
+//    queues a fingerprint check of the lists (fgms_plan_check), and the call after
+//    a rewrite raises RuntimeError and drops the plan.  A call with in_map and out_map exchanged (the
 //    transposed convolution over the same pairs) shares the cached plan's tables;
 //  * HIP errors raise RuntimeError instead of passing silently.
 #include <torch/extension.h>
@@ -105,6 +106,19 @@ fgms_plan_t *plan_for(const at::Tensor &kpos, const at::Tensor &in_map, const at
         it->n_in == n_in && it->n_out == n_out && it->device == dev) {
       if (it->v_in == version_of(in_map) && it->v_out == version_of(out_map) &&
           it->v_kpos == version_of(kpos)) {
+        // The version counters do not see writes through raw pointers (a map builder filling a
+        // pre-allocated tensor, this library's own included).  Every hit queues a check of the
+        // lists against the fingerprint the plan was built with; what it finds reaches the host
+        // a call later: that call drops the plan and raises.
+        const int rc = fgms_plan_check(it->plan, stream, 1);      // (rides along with this call's launch)
+        if (rc == FGMS_E_STALE) {
+          drop(it);
+          throw std::runtime_error(
+              "FGMS: the kernel map tensors were rewritten in place after their plan was cached "
+              "(a write through data_ptr() does not bump the version counter); the previous call on this "
+              "map used the old neighbour tables.  Call fgms_plan_cache_clear() after rewriting a map.");
+        }
+        check(rc);
         g_cache.splice(g_cache.begin(), g_cache, it);
         return g_cache.front().plan;
       }

@@ -53,6 +53,7 @@ extern "C" {
 #define FGMS_E_INVALID (-1)   /* bad argument (shape, dtype, null pointer)   */
 #define FGMS_E_HIP (-2)       /* a HIP runtime call failed                    */
 #define FGMS_E_NOMEM (-3)     /* workspace / plan allocation failed           */
+#define FGMS_E_STALE (-4)     /* the pair lists changed after the plan was made */
 
 typedef struct fgms_plan fgms_plan_t;
 
@@ -90,6 +91,22 @@ int fgms_plan_create(fgms_plan_t **plan, const int32_t *kpos,
  */
 int fgms_plan_transposed(fgms_plan_t **view, fgms_plan_t *base);
 void fgms_plan_destroy(fgms_plan_t *plan);
+/*
+ * Guards against a plan that outlived its map (no counterpart in the reference, which reads
+ * the pair lists on every call, backend/spconv.cuh:484-485, and so cannot compute with last
+ * iteration's neighbours).  The build keeps a fingerprint of the lists: kpos and a fixed
+ * sample of about 4 096 (in_map, out_map) entries.  fgms_plan_check has the fingerprint taken
+ * again from the lists as they are then: by one small kernel queued on `stream` right away
+ * (with_next_launch = 0), or by one extra workgroup of the next forward / backward launch
+ * that reads the plan (with_next_launch = 1: no launch of its own, `stream` is not used).  A
+ * difference raises a flag in the plan, and every later call that is handed the plan (this
+ * one included) returns FGMS_E_STALE once the flag has reached the host.  The check does not
+ * wait for the GPU, so the call that carried it may still have computed with the old tables:
+ * a caller that rewrites its lists in place must make a new plan; this only makes the
+ * omission loud.  A sample is not a proof: rewrites that leave kpos and every sampled entry
+ * as they were go unnoticed.
+ */
+int fgms_plan_check(fgms_plan_t *plan, void *stream, int with_next_launch);
 /* 1 if the output-stationary kernels can use it for forward / for dgrad. */
 int fgms_plan_usable(const fgms_plan_t *plan, int for_dgrad);
 /* What the build counted (no counterpart in the reference): stats[0] = pairs in the map,
@@ -171,8 +188,11 @@ int fgms_wgrad(const void *in_feats, const void *out_feats_grad, void *kernel_gr
  * k_vol * c_in * c_out <= 2 097 152 (27 offsets of 256 x 256 fit); only the shapes of the
  * MFMA and skinny kernels (channel counts that are multiples of 32, or 4/8/16 -> 16/32/64,
  * 16-byte aligned rows) -- anything else returns FGMS_E_INVALID instead of falling back to a
- * kernel that would need a workspace.  All calls on one GPU share that GPU's array: calls
- * that overlap in time on one GPU (two streams, two threads) race; calls on one stream do not.
+ * kernel that would need a workspace.  A plan is used only if an earlier call has already
+ * taken its build results (the first use of a plan waits for the build and may allocate);
+ * otherwise the call runs without the plan's row bands.  All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls
+ * on one stream do not.
  */
 int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *kernel_grad,
                       const int32_t *kpos, const int32_t *in_map, const int32_t *out_map,

@@ -57,6 +57,9 @@ int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad,
  * index-th record: kernel name and milliseconds; it returns FGMS_E_INVALID
  * once index runs past the records.  fgms_profile_reset drops all records.
  */
+/* How many device or pinned-host allocations (hipMalloc, hipHostMalloc) the library has made
+ * since it was loaded: a test can assert that a call made none. */
+long long fgms_allocation_count(void);
 void fgms_profile_enable(int on);
 int fgms_profile_read(int index, char *name, int name_len, float *ms);
 void fgms_profile_reset(void);

@@ -89,3 +89,38 @@ def test_small_launches_on_256_row_tiles():
     tiles and this one through the others; both meet the oracle)."""
     names = run_child({"FGMS_HALF_TILES": "0"})
     assert "bwd_fused_kernel" in names and "gms_rows_kernel(fwd)" in names, names
+
+
+FULL_SIZE_CHILD = r"""
+import sys
+import numpy as np, torch
+sys.path.insert(0, %r)
+import bench
+from fgms_amd import capi
+from oracle import fgms_oracle as oracle
+from tests import gpu_util as G
+L, passes, arch80 = bench.make_case("cfg2-indoor200k-k27-64x64-tf32-fwd", 1.0)
+assert arch80 and L["in_feats"].dtype == np.float32 and L["n_in"] >= 190000
+D = G.to_dev(L)
+plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+capi.profile_reset(); capi.profile_enable(True)
+out = G.run_fwd(capi, D, fused=True, arch80=True, plan=plan)
+capi.profile_enable(False)
+names = sorted({n for n, _ in capi.profile_records()})
+want = oracle.c_fwd(L["in_feats"], L["kernel"], L["knnz"], L["imap"], L["omap"], L["n_out"])
+G.assert_close(out, want, "tf32", "cfg2 at full size, tf32 mode on fp32 matrix instructions")
+G.assert_close(out, want, "fp32", "the same, held to the fp32 tolerance (the arithmetic is fp32)")
+print("KERNELS " + " ".join(names))
+""" % ROOT
+
+
+def test_tf32_mode_on_fp32_matrix_instructions_at_full_size():
+    """The arithmetic the task prescribes for tf32 mode (fp32 MFMA, FGMS_SPLIT_BF16=0) on the
+    200 000-voxel cloud of BASELINE config 2, element by element against the C oracle."""
+    env = dict(os.environ)
+    env["FGMS_SPLIT_BF16"] = "0"
+    r = subprocess.run([sys.executable, "-c", FULL_SIZE_CHILD], env=env, cwd=ROOT, stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("KERNELS ")][-1]
+    assert "bf16x3" not in line and "gms_rows_kernel(fwd)" in line, line

@@ -558,3 +558,33 @@ def test_tf32_mode_without_a_plan(capi, oracle, shape):
     for fused in (True, False):
         G.assert_close(G.run_fwd(capi, Ds, fused=fused, separate_mid=True, arch80=True, plan=None), ref, "tf32",
                        "tf32-mode forward, centre apart")
+
+
+@pytest.mark.parametrize("shape", [(32, 32), (64, 64)], ids=["32x32", "64x64"])
+def test_fp32_with_half_the_rms_floor(capi, oracle, shape):
+    """assert_close allows rtol * rms(reference) on top of the relative bound, which for
+    small-magnitude elements is most of the allowance.  Here the fp32 path is held to
+    |d| <= 1e-5 |ref| + 5e-6 rms(ref) against the float64 formulation, half the usual floor, and
+    the error of the typical element to a tenth of it.  (A sum of a thousand fp32 products
+    carries rounding noise of 2-3e-6 of the result's rms in its worst elements, whatever the
+    order of summation: a floor below that would test the number format, not the kernel.)"""
+    L = layer(43, shape[0], shape[1], np.float32)
+    D = G.to_dev(L)
+    args = (L["knnz"], L["imap"], L["omap"])
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+
+    def tight(got, ref, what):
+        got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+        rms = float(np.sqrt(np.mean(ref ** 2)))
+        err = np.abs(got - ref)
+        bad = err > 1e-5 * np.abs(ref) + 5e-6 * rms
+        assert not bad.any(), "%s: %d / %d outside 1e-5 |ref| + 5e-6 rms (worst %.3g of rms)" % (
+            what, int(bad.sum()), bad.size, float(err.max() / rms))
+        assert float(np.median(err)) <= 1e-6 * rms, (what, float(np.median(err)) / rms)
+
+    for p, tag in ((plan, "plan"), (None, "no plan")):
+        tight(G.run_fwd(capi, D, plan=p), oracle.np_fwd(L["in_feats"], L["kernel"], *args, L["n_out"]), "fwd, " + tag)
+        gi, gw = G.run_bwd(capi, D, plan=p)
+        tight(gi, oracle.np_dgrad(L["out_grad"], L["kernel"], *args, L["n_in"]), "dgrad, " + tag)
+        tight(gw, oracle.np_wgrad(L["in_feats"], L["out_grad"], *args, L["k_vol"]), "wgrad, " + tag)
+    plan.close()

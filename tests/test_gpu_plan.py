@@ -170,3 +170,97 @@ def test_more_than_64_offsets_keep_the_output_stationary_kernels(capi, oracle, d
     out_seq = G.run_fwd(capi, D, fused=False, plan=plan)
     G.assert_close(out_seq, out.astype(np.float32), mode, "seq fwd")
     plan.close()
+
+
+def _two_clouds(n=6000):
+    a = clouds.cloud_indoor(clouds.rng_for(2), target=n)
+    b = clouds.cloud_indoor(clouds.rng_for(7), target=n)
+    m = min(len(a), len(b))
+    return np.ascontiguousarray(a[:m], dtype=np.int32), np.ascontiguousarray(b[:m], dtype=np.int32)
+
+
+def test_rewritten_map_is_noticed_by_the_plan(capi, oracle):
+    """A map rewritten through raw pointers (how a native builder fills a pre-allocated tensor)
+    leaves the plan with last iteration's neighbour tables.  fgms_plan_check queues a
+    fingerprint check; the call after it raises."""
+    va, vb = _two_clouds()
+    offs = clouds.offsets_cube(3)
+    n, k_vol = len(va), len(offs)
+    cap = n * k_vol
+    into = (torch.empty(cap, dtype=torch.int32, device="cuda"), torch.empty(cap, dtype=torch.int32, device="cuda"),
+            torch.empty(k_vol, dtype=torch.int32, device="cuda"), torch.empty(k_vol + 1, dtype=torch.int32, device="cuda"))
+    ca, cb = torch.from_numpy(va).cuda(), torch.from_numpy(vb).cuda()
+    imap, omap, knnz, kpos = capi.build_kernel_map(ca, ca, offs, 1, into=into)
+    plan = capi.Plan(kpos, imap, omap, n, n)
+    plan.check(); plan.check()
+    torch.cuda.synchronize()
+    plan.check()                                  # unchanged lists: nothing to report
+    capi.build_kernel_map(cb, cb, offs, 1, into=into)      # same tensors, new content
+    plan.check()                                  # queues the check that finds it
+    torch.cuda.synchronize()
+    with pytest.raises(capi.StalePlanError):
+        plan.check()
+    x = torch.zeros(n, 32, dtype=torch.float16, device="cuda")
+    w = torch.zeros(k_vol, 32, 32, dtype=torch.float16, device="cuda")
+    out = torch.zeros(n, 32, dtype=torch.float16, device="cuda")
+    with pytest.raises(capi.StalePlanError):      # every entry point refuses the plan from now on
+        capi.fusion_fwd(x, w, 0, out, kpos, None, imap, omap, False, False, plan=plan)
+    plan.close()
+    # the same with the check carried by the forward / backward launches themselves
+    g = torch.zeros(n, 32, dtype=torch.float16, device="cuda")
+    gi, gw = torch.zeros_like(x), torch.zeros_like(w)
+    for use in ("fwd", "bwd"):
+        capi.build_kernel_map(ca, ca, offs, 1, into=into)
+        plan = capi.Plan(kpos, imap, omap, n, n)
+
+        def call():
+            plan.check(with_next_launch=True)
+            if use == "fwd":
+                capi.fusion_fwd(x, w, 0, out, kpos, None, imap, omap, False, False, plan=plan)
+            else:
+                capi.bwd(g, x, w, 0, gi, gw, kpos, None, imap, omap, False, False, plan=plan)
+            torch.cuda.synchronize()
+
+        call(); call()
+        capi.build_kernel_map(cb, cb, offs, 1, into=into)
+        call()                                    # old tables; the launch's extra workgroup notices
+        with pytest.raises(capi.StalePlanError):
+            call()
+        plan.close()
+
+
+def test_backend_cache_drops_a_plan_whose_map_was_rewritten(capi, oracle):
+    import FGMS.backend as backend
+    backend.fgms_plan_cache(True)
+    backend.fgms_plan_cache_clear()
+    va, vb = _two_clouds()
+    offs = clouds.offsets_cube(3)
+    n, k_vol = len(va), len(offs)
+    cap = n * k_vol
+    into = (torch.empty(cap, dtype=torch.int32, device="cuda"), torch.empty(cap, dtype=torch.int32, device="cuda"),
+            torch.empty(k_vol, dtype=torch.int32, device="cuda"), torch.empty(k_vol + 1, dtype=torch.int32, device="cuda"))
+    rng = np.random.default_rng(3)
+    x_np = rng.standard_normal((n, 32)).astype(np.float16)
+    w_np = (rng.standard_normal((k_vol, 32, 32)) * 0.1).astype(np.float16)
+    x, w = torch.from_numpy(x_np).cuda(), torch.from_numpy(w_np).cuda()
+
+    def forward():
+        out = torch.zeros(n, 32, dtype=torch.float16, device="cuda")
+        backend.fgms_fusion_fwd_cuda(x, w, 0, out, into[3], torch.zeros_like(into[3]), into[0], into[1], False, False)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    def reference():
+        kp = into[3].cpu().numpy()
+        m = int(kp[-1])
+        return oracle.c_fwd(x_np, w_np, into[2].cpu().numpy(), into[0][:m].cpu().numpy(), into[1][:m].cpu().numpy(), n)
+
+    capi.build_kernel_map(torch.from_numpy(va).cuda(), torch.from_numpy(va).cuda(), offs, 1, into=into)
+    G.assert_close(forward(), reference(), "fp16", "first map")
+    G.assert_close(forward(), reference(), "fp16", "first map, plan from the cache")
+    capi.build_kernel_map(torch.from_numpy(vb).cuda(), torch.from_numpy(vb).cuda(), offs, 1, into=into)
+    forward()                                     # computes with the old tables; its check notices
+    with pytest.raises(RuntimeError, match="rewritten in place"):
+        forward()
+    G.assert_close(forward(), reference(), "fp16", "second map, after the stale plan was dropped")
+    backend.fgms_plan_cache_clear()

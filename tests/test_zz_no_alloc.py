@@ -69,3 +69,32 @@ def test_static_weight_gradient_accumulates_and_rejects(capi):
     g = torch.zeros(D["n_out"], 40, dtype=torch.float16, device="cuda")
     with pytest.raises(ValueError, match="only the shapes"):
         capi.wgrad_static(x, g, odd_w, D["kpos"], D["imap"], D["omap"])
+
+
+def test_static_weight_gradient_allocates_nothing(capi):
+    """The entry point's defining property: no device or pinned allocation, also when it is
+    the first call to see a fresh plan of a strided (sparse) map -- taking that plan's build
+    results would wait for the build and may allocate its pair view, so the call does without."""
+    rng = np.random.default_rng(12)
+    vin = clouds.cloud_indoor(clouds.rng_for(2), target=20000)
+    vout = clouds.downsample_coords(vin, 2)
+    imap, omap, knnz, kpos = clouds.build_kernel_map(vin, vout, clouds.offsets_cube(2), stride=2)
+    L = clouds.make_layer(rng, imap, omap, knnz, kpos, len(vin), len(vout), 64, 128, np.float16)
+    D = G.to_dev(L)
+    got = torch.zeros_like(D["kernel"])
+    capi.wgrad_static(D["in_feats"], D["out_grad"], got, D["kpos"], D["imap"], D["omap"])       # warm-up: symbol address, LDS limits
+    torch.cuda.synchronize()
+    plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])                  # (the build allocates; the call below must not)
+    torch.cuda.synchronize()
+    before, free_before = capi.allocation_count(), torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        got.zero_()
+        capi.wgrad_static(D["in_feats"], D["out_grad"], got, D["kpos"], D["imap"], D["omap"], plan=plan)
+    torch.cuda.synchronize()
+    assert capi.allocation_count() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
+    want = torch.zeros_like(D["kernel"])
+    capi.wgrad(D["in_feats"], D["out_grad"], want, D["kpos"], D["imap"], D["omap"], plan=plan)
+    torch.cuda.synchronize()
+    G.assert_close(got.cpu().numpy(), want.cpu().numpy(), "fp16", "static (fresh plan of a strided map) vs fgms_wgrad")
+    plan.close()
