@@ -121,8 +121,8 @@ __device__ __forceinline__ void add_and_clear_elements(__half *__restrict__ dst,
 
 // Fingerprint of the pair lists: the sum, over a fixed sample of positions (every `stride`-th
 // pair) and over kpos, of a hash of (position, values).  Taken by the build (inside
-// pair_masks_kernel) and again by fgms_plan_check; sums of 64-bit hashes, so the order in which
-// threads add does not matter.
+// pair_masks_kernel's launch) and again by fgms_plan_check; sums of 64-bit hashes, so the order
+// in which threads add does not matter.
 __device__ __forceinline__ unsigned long long print_hash(unsigned long long a, unsigned b, unsigned c) {
   unsigned long long x = a * 0x9E3779B97F4A7C15ull + ((unsigned long long)b << 32 | c);
   x ^= x >> 31; x *= 0xBF58476D1CE4E5B9ull; x ^= x >> 29;
@@ -131,48 +131,60 @@ __device__ __forceinline__ unsigned long long print_hash(unsigned long long a, u
 constexpr int kPrintSamples = 4096;
 __host__ __device__ inline int print_stride(int n_pairs) { return n_pairs > kPrintSamples ? n_pairs / kPrintSamples : 1; }
 
-// This thread's share of the fingerprint: pair j if it is a sampled one, and entry j - first of
-// kpos for the first k_vol + 1 pairs.  (first = kpos[0], total = pairs in the lists.)
-__device__ __forceinline__ unsigned long long print_share(const int32_t *__restrict__ kpos,
-                                                          const int32_t *__restrict__ imap,
-                                                          const int32_t *__restrict__ omap, int k_vol,
-                                                          int first, int total, int j) {
-  unsigned long long v = 0;
-  const int rel = j - first, stride = print_stride(total - first);
-  if (rel % stride == 0) v += print_hash((unsigned long long)rel, (unsigned)imap[j], (unsigned)omap[j]);
-  if (rel <= k_vol) v += print_hash(0x100000000ull + rel, (unsigned)kpos[rel], 0u);
-  return v;
-}
-
-
-// The fingerprint taken again from the lists as they are now, by one workgroup (the sample is
-// 4 096 pairs), and compared with the build's; a difference raises the sticky flag, in device
-// memory and in the plan's pinned block (fgms_plan_check).
-__device__ __forceinline__ void plan_check_block(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-                                                 const int32_t *__restrict__ omap, int k_vol, int n_pairs,
-                                                 int *__restrict__ flags, int *__restrict__ host) {
+// The fingerprint of the lists as they are now, summed by one workgroup (the sample is 4 096
+// pairs); valid in thread 0.
+__device__ __forceinline__ unsigned long long plan_print_sum(const int32_t *__restrict__ kpos,
+                                                             const int32_t *__restrict__ imap,
+                                                             const int32_t *__restrict__ omap, int k_vol, int n_pairs) {
   __shared__ unsigned long long part[16];
   const int threads = blockDim.x;
   const int first = kpos[0], total = min(kpos[k_vol], n_pairs);
   const int stride = print_stride(total - first);
   unsigned long long v = 0;
-  // the sampled pairs, then the pairs whose threads carried kpos in the build
-  for (int s = threadIdx.x; first + (long long)s * stride < total; s += threads) {
-    const int j = first + s * stride;
-    v += print_hash((unsigned long long)(j - first), (unsigned)imap[j], (unsigned)omap[j]);
+  // (all of a thread's samples are requested before the first is hashed)
+  constexpr int kMine = 16;
+  for (int s0 = threadIdx.x; first + (long long)s0 * stride < total; s0 += threads * kMine) {
+    int a[kMine], b[kMine];
+#pragma unroll
+    for (int u = 0; u < kMine; ++u) {
+      const long long j = first + (long long)(s0 + u * threads) * stride;
+      const int jj = (int)(j < total ? j : total - 1);
+      a[u] = imap[jj];
+      b[u] = omap[jj];
+    }
+#pragma unroll
+    for (int u = 0; u < kMine; ++u) {
+      const long long j = first + (long long)(s0 + u * threads) * stride;
+      if (j < total) v += print_hash((unsigned long long)(j - first), (unsigned)a[u], (unsigned)b[u]);
+    }
   }
-  for (int rel = threadIdx.x; rel <= k_vol && first + rel < total; rel += threads)
-    v += print_hash(0x100000000ull + rel, (unsigned)kpos[rel], 0u);
+  for (int rel = threadIdx.x; rel <= k_vol; rel += threads) v += print_hash(0x100000000ull + rel, (unsigned)kpos[rel], 0u);
   for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
   if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = v;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned long long sum = 0;
+  unsigned long long sum = 0;
+  if (threadIdx.x == 0)
     for (int w = 0; w < threads / 64; ++w) sum += part[w];
-    if (sum != *reinterpret_cast<const unsigned long long *>(flags + kFlagPrint)) {
-      flags[kFlagStale] = 1;
-      if (host) host[kFlagStale] = 1;
-    }
+  return sum;
+}
+
+// Build: the fingerprint goes into the plan's flags.
+__device__ __forceinline__ void plan_print_block(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+                                                 const int32_t *__restrict__ omap, int k_vol, int n_pairs,
+                                                 int *__restrict__ flags) {
+  const unsigned long long sum = plan_print_sum(kpos, imap, omap, k_vol, n_pairs);
+  if (threadIdx.x == 0) *reinterpret_cast<unsigned long long *>(flags + kFlagPrint) = sum;
+}
+
+// fgms_plan_check: taken again and compared with the build's; a difference raises the sticky
+// flag, in device memory and in the plan's pinned block.
+__device__ __forceinline__ void plan_check_block(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+                                                 const int32_t *__restrict__ omap, int k_vol, int n_pairs,
+                                                 int *__restrict__ flags, int *__restrict__ host) {
+  const unsigned long long sum = plan_print_sum(kpos, imap, omap, k_vol, n_pairs);
+  if (threadIdx.x == 0 && sum != *reinterpret_cast<const unsigned long long *>(flags + kFlagPrint)) {
+    flags[kFlagStale] = 1;
+    if (host) host[kFlagStale] = 1;
   }
 }
 

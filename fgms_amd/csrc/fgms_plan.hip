@@ -28,6 +28,17 @@ __global__ void fill_i32_kernel(int32_t *__restrict__ p, size_t n, int32_t v) {
   if (i < n % 4) p[n4 * 4 + i] = v;
 }
 
+// Two fills in one launch (the build is a chain of small launches, each bound by its latency).
+__global__ void fill_two_kernel(int32_t *__restrict__ p1, size_t n1, int32_t v1, int32_t *__restrict__ p2, size_t n2,
+                                int32_t v2) {
+  typedef int int4v_ __attribute__((ext_vector_type(4)));
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t q = i; q < n1 / 4; q += stride) reinterpret_cast<int4v_ *>(p1)[q] = int4v_{v1, v1, v1, v1};
+  if (i < n1 % 4) p1[n1 / 4 * 4 + i] = v1;
+  for (size_t q = i; q < n2 / 4; q += stride) reinterpret_cast<int4v_ *>(p2)[q] = int4v_{v2, v2, v2, v2};
+  if (i < n2 % 4) p2[n2 / 4 * 4 + i] = v2;
+}
+
 // flags[0]: an index is out of range; flags[1]: two pairs of one offset share
 // an output row; flags[2]: two pairs of one offset share an input row;
 // flags[3]: inside some offset the pairs are not ordered by output row;
@@ -45,7 +56,13 @@ __global__ void pair_masks_kernel(const int32_t *__restrict__ kpos, const int32_
                                   int n_out, unsigned long long *__restrict__ rmask_out,
                                   unsigned long long *__restrict__ rmask_in, int *__restrict__ flags) {
   const int total = kpos[k_vol];
-  const int j = kpos[0] + blockIdx.x * blockDim.x + threadIdx.x;      // (kpos[0] > 0: a plan over a slice of the offsets)
+  if (blockIdx.x == 0) {
+    // the launch's first workgroup takes the fingerprint of the lists (fgms_plan_check re-takes
+    // it); first, so that its chain of loads runs next to the others' work, not behind it
+    plan_print_block(kpos, imap, omap, k_vol, n_pairs, flags);
+    return;
+  }
+  const int j = kpos[0] + (blockIdx.x - 1) * blockDim.x + threadIdx.x;      // (kpos[0] > 0: a plan over a slice of the offsets)
   if (j >= total || j >= n_pairs) return;
   int lo = 0, hi = k_vol;          // offset of pair j: the last k with kpos[k] <= j
   while (hi - lo > 1) {
@@ -55,10 +72,6 @@ __global__ void pair_masks_kernel(const int32_t *__restrict__ kpos, const int32_
   const int k = lo;
   const int i = imap[j], o = omap[j];
   if (j == kpos[0]) flags[12] = min(total, n_pairs) - kpos[0];
-  {
-    const unsigned long long share = print_share(kpos, imap, omap, k_vol, kpos[0], min(total, n_pairs), j);
-    if (share) atomicAdd(reinterpret_cast<unsigned long long *>(flags + kFlagPrint), share);
-  }
   if (i < 0 || i >= n_in || o < 0 || o >= n_out) {
     flags[0] = 1;
     return;
@@ -270,13 +283,13 @@ __global__ __launch_bounds__(kSortThreads) void sort_window_kernel(SortArgs a) {
 
 // Step 3: the neighbour tables by POSITION, straight from the pair lists (tables pre-filled
 // with -1): nbr_out[k][position of o] = i, nbr_in[k][position of i] = o.
-__global__ void tables_kernel(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
-                              const int32_t *__restrict__ omap, int k_vol, int n_pairs, int n_in,
-                              int n_out, const int32_t *__restrict__ inv_out,
-                              const int32_t *__restrict__ inv_in, int32_t *__restrict__ nbr_out,
-                              int32_t *__restrict__ nbr_in) {
+__device__ __forceinline__ void tables_body(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+                                            const int32_t *__restrict__ omap, int k_vol, int n_pairs, int n_in,
+                                            int n_out, const int32_t *__restrict__ inv_out,
+                                            const int32_t *__restrict__ inv_in, int32_t *__restrict__ nbr_out,
+                                            int32_t *__restrict__ nbr_in, int block) {
   const int total = kpos[k_vol];
-  const int j = kpos[0] + blockIdx.x * blockDim.x + threadIdx.x;
+  const int j = kpos[0] + block * blockDim.x + threadIdx.x;
   if (j >= total || j >= n_pairs) return;
   int lo = 0, hi = k_vol;
   while (hi - lo > 1) {
@@ -333,6 +346,13 @@ __global__ __launch_bounds__(1024) void block_masks_kernel(MaskArgs a) {
     if (sum) atomicAdd(&a.flags[4 + blockIdx.y], sum);
     if (rows) atomicAdd(&a.flags[10 + blockIdx.y], rows);
   }
+}
+
+__global__ void tables_kernel(const int32_t *__restrict__ kpos, const int32_t *__restrict__ imap,
+                              const int32_t *__restrict__ omap, int k_vol, int n_pairs, int n_in, int n_out,
+                              const int32_t *__restrict__ inv_out, const int32_t *__restrict__ inv_in,
+                              int32_t *__restrict__ nbr_out, int32_t *__restrict__ nbr_in) {
+  tables_body(kpos, imap, omap, k_vol, n_pairs, n_in, n_out, inv_out, inv_in, nbr_out, nbr_in, blockIdx.x);
 }
 
 // Pair view: the pair lists with every offset's run padded to a multiple of 64 rows
@@ -416,6 +436,8 @@ struct TileSide {
 struct TileArgs {
   TileSide side[2];
   int cus_per_xcd;
+  const int *flags;   // the build's findings and where they go on the host (this is the
+  int *host;          // build's last launch); nullptr: published by a launch of its own
 };
 __global__ __launch_bounds__(1024) void tile_order_kernel(TileArgs ta) {
   const int32_t *__restrict__ perm = ta.side[blockIdx.x].perm;
@@ -423,6 +445,7 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(TileArgs ta) {
   int32_t *__restrict__ order = ta.side[blockIdx.x].order;
   const int n_rows = ta.side[blockIdx.x].n_rows, n_tiles = ta.side[blockIdx.x].n_tiles;
   const int cap = ta.side[blockIdx.x].cap, cus_per_xcd = ta.cus_per_xcd;
+  if (blockIdx.x == 0 && ta.host && threadIdx.x < kPlanFlags) ta.host[threadIdx.x] = ta.flags[threadIdx.x];
   if (!order) return;
   constexpr int kPc = 65;                         // popcount classes 0..64
   __shared__ int hist[8][kPc];                    // tiles per (home, popcount), then start ranks
@@ -703,7 +726,8 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
     p->mask_in = p->mask_out + bo;
   }
   unsigned long long *rmask_out = rmask, *rmask_in = rmask ? rmask + n_out : nullptr;
-  if ((rc = fill_i32(p->flags, kPlanFlags, 0, s))) return fail(rc);
+  // (the flags are cleared together with the row masks below; without tables, here)
+  if (!tables && (rc = fill_i32(p->flags, kPlanFlags, 0, s))) return fail(rc);
   p->has_tables = tables;
   p->has_bands = want_bands;
 
@@ -747,22 +771,25 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
       return fail(FGMS_E_HIP);
     }
   }
+  if (tables) {
+    const size_t n_mask = (size_t)(n_out + n_in) * 2;
+    size_t blocks = (n_mask / 4 + 255) / 256;
+    fill_two_kernel<<<(unsigned)(blocks > 8192 ? 8192 : (blocks ? blocks : 1)), 256, 0, s>>>(
+        (int32_t *)rmask, n_mask, 0, p->flags, (size_t)kPlanFlags, 0);
+    if (hipGetLastError() != hipSuccess) {
+      drop_events();
+      set_error("fgms_plan_create: a build launch failed");
+      return fail(FGMS_E_HIP);
+    }
+  }
   if (tables && n_pairs > 0) {
-    if ((rc = fill_i32((int32_t *)rmask, (size_t)(n_out + n_in) * 2, 0, s))) {
-      drop_events();
-      return fail(rc);
-    }
-    pair_masks_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
+    pair_masks_kernel<<<(unsigned)((n_pairs + 255) / 256) + 1, 256, 0, s>>>(
         kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, rmask_out, rmask_in, p->flags);
-  } else if (tables) {
-    if ((rc = fill_i32((int32_t *)rmask, (size_t)(n_out + n_in) * 2, 0, s))) {
-      drop_events();
-      return fail(rc);
-    }
   }
   // row orders (both sides in the same launches)
   static const bool sort_rows = !(getenv("FGMS_PLAN_SORT") && atoi(getenv("FGMS_PLAN_SORT")) == 0);
   int32_t *inv[2] = {nullptr, nullptr};
+  bool published = false;      // the flags reach the host with the tile-order launch
   if (tables) {
     SortArgs sa{};
     sa.k_vol = k_vol;
@@ -820,15 +847,31 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   }
   drop_events();
   if (tables) {
-    if (n_pairs > 0)
-      tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
-          kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, inv[0], inv[1], p->nbr_out, p->nbr_in);
     MaskArgs ma{};
     ma.flags = p->flags;
     ma.side[0] = MaskSide{rmask_out, p->perm_out, p->mask_out, (int)n_out};
     ma.side[1] = MaskSide{rmask_in, p->perm_in, p->mask_in, (int)n_in};
     const size_t most = bo > bi ? bo : bi;
-    if (most > 0) block_masks_kernel<<<dim3((unsigned)((most + 15) / 16), 2), 1024, 0, s>>>(ma);
+    // second fork: the block masks and the tile order need the row order only, not the tables;
+    // they run on the side stream next to the table writes (each of these launches is bound by
+    // its latency and by the gap to the next one)
+    hipEvent_t sorted = nullptr, masked = nullptr;
+    hipStream_t sm = s;
+    if (s2 && most > 0 && n_pairs > 0) {
+      if (hipEventCreateWithFlags(&sorted, hipEventDisableTiming) == hipSuccess &&
+          hipEventCreateWithFlags(&masked, hipEventDisableTiming) == hipSuccess &&
+          hipEventRecord(sorted, s) == hipSuccess && hipStreamWaitEvent(s2, sorted, 0) == hipSuccess) {
+        sm = s2;
+      } else {
+        if (sorted) (void)hipEventDestroy(sorted);
+        if (masked) (void)hipEventDestroy(masked);
+        sorted = masked = nullptr;
+      }
+    }
+    if (n_pairs > 0)
+      tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
+          kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, inv[0], inv[1], p->nbr_out, p->nbr_in);
+    if (most > 0) block_masks_kernel<<<dim3((unsigned)((most + 15) / 16), 2), 1024, 0, sm>>>(ma);
     // tile -> XCD homes pay off once every XCD has a few dozen tiles of its own
     static const bool xcd_homes = !(getenv("FGMS_XCD_HOME") && atoi(getenv("FGMS_XCD_HOME")) == 0);
     TileArgs ta{};
@@ -840,12 +883,26 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
       if (!xcd_homes || n_tiles < 256 || (size_t)n_tiles * sizeof(int32_t) > 60000) continue;
       int32_t *&order = d ? p->tile_in : p->tile_out;
       const int cap = (n_tiles + 7) / 8;
-      if (!take((void **)&order, (size_t)cap * 8 * sizeof(int32_t), false)) return fail(FGMS_E_NOMEM);
+      if (!take((void **)&order, (size_t)cap * 8 * sizeof(int32_t), false)) {
+        order = nullptr;       // (the kernels then take the tiles in plain order)
+        continue;
+      }
       (d ? p->tile_grid_in : p->tile_grid_out) = cap * 8;
       ta.side[d] = TileSide{d ? p->perm_in : p->perm_out, d ? p->mask_in : p->mask_out, order, (int)n, n_tiles, cap};
       if (n_tiles > most_tiles) most_tiles = n_tiles;
     }
-    if (most_tiles > 0) tile_order_kernel<<<2, 1024, (size_t)most_tiles * sizeof(int32_t), s>>>(ta);
+    if (most_tiles > 0) {
+      if (hipHostGetDevicePointer((void **)&ta.host, p->host_flags, 0) != hipSuccess) ta.host = nullptr;
+      ta.flags = p->flags;
+      tile_order_kernel<<<2, 1024, (size_t)most_tiles * sizeof(int32_t), sm>>>(ta);
+      published = ta.host != nullptr;
+    }
+    if (sm != s) {
+      const bool ok = hipEventRecord(masked, sm) == hipSuccess && hipStreamWaitEvent(s, masked, 0) == hipSuccess;
+      if (!ok) (void)hipStreamSynchronize(sm);
+      (void)hipEventDestroy(sorted);
+      (void)hipEventDestroy(masked);
+    }
   }
   if (hipGetLastError() != hipSuccess) {
     set_error("fgms_plan_create: a build launch failed");
@@ -853,7 +910,7 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
   }
   int *host_dev = nullptr;
   if (hipHostGetDevicePointer((void **)&host_dev, p->host_flags, 0) != hipSuccess) host_dev = nullptr;
-  if (host_dev) publish_flags_kernel<<<1, 64, 0, s>>>(p->flags, host_dev);
+  if (host_dev && !published) publish_flags_kernel<<<1, 64, 0, s>>>(p->flags, host_dev);
   if ((!host_dev && hipMemcpyAsync(p->host_flags, p->flags, kPlanFlags * sizeof(int), hipMemcpyDeviceToHost, s) != hipSuccess) ||
       hipEventRecord(p->ready, s) != hipSuccess) {
     set_error("fgms_plan_create: queuing the flag read-back failed");
