@@ -852,26 +852,10 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
     ma.side[0] = MaskSide{rmask_out, p->perm_out, p->mask_out, (int)n_out};
     ma.side[1] = MaskSide{rmask_in, p->perm_in, p->mask_in, (int)n_in};
     const size_t most = bo > bi ? bo : bi;
-    // second fork: the block masks and the tile order need the row order only, not the tables;
-    // they run on the side stream next to the table writes (each of these launches is bound by
-    // its latency and by the gap to the next one)
-    hipEvent_t sorted = nullptr, masked = nullptr;
-    hipStream_t sm = s;
-    if (s2 && most > 0 && n_pairs > 0) {
-      if (hipEventCreateWithFlags(&sorted, hipEventDisableTiming) == hipSuccess &&
-          hipEventCreateWithFlags(&masked, hipEventDisableTiming) == hipSuccess &&
-          hipEventRecord(sorted, s) == hipSuccess && hipStreamWaitEvent(s2, sorted, 0) == hipSuccess) {
-        sm = s2;
-      } else {
-        if (sorted) (void)hipEventDestroy(sorted);
-        if (masked) (void)hipEventDestroy(masked);
-        sorted = masked = nullptr;
-      }
-    }
     if (n_pairs > 0)
       tables_kernel<<<(unsigned)((n_pairs + 255) / 256), 256, 0, s>>>(
           kpos, in_map, out_map, k_vol, (int)n_pairs, (int)n_in, (int)n_out, inv[0], inv[1], p->nbr_out, p->nbr_in);
-    if (most > 0) block_masks_kernel<<<dim3((unsigned)((most + 15) / 16), 2), 1024, 0, sm>>>(ma);
+    if (most > 0) block_masks_kernel<<<dim3((unsigned)((most + 15) / 16), 2), 1024, 0, s>>>(ma);
     // tile -> XCD homes pay off once every XCD has a few dozen tiles of its own
     static const bool xcd_homes = !(getenv("FGMS_XCD_HOME") && atoi(getenv("FGMS_XCD_HOME")) == 0);
     TileArgs ta{};
@@ -894,14 +878,8 @@ int plan_create(fgms_plan_t **plan_out, const int32_t *kpos, const int32_t *in_m
     if (most_tiles > 0) {
       if (hipHostGetDevicePointer((void **)&ta.host, p->host_flags, 0) != hipSuccess) ta.host = nullptr;
       ta.flags = p->flags;
-      tile_order_kernel<<<2, 1024, (size_t)most_tiles * sizeof(int32_t), sm>>>(ta);
+      tile_order_kernel<<<2, 1024, (size_t)most_tiles * sizeof(int32_t), s>>>(ta);
       published = ta.host != nullptr;
-    }
-    if (sm != s) {
-      const bool ok = hipEventRecord(masked, sm) == hipSuccess && hipStreamWaitEvent(s, masked, 0) == hipSuccess;
-      if (!ok) (void)hipStreamSynchronize(sm);
-      (void)hipEventDestroy(sorted);
-      (void)hipEventDestroy(masked);
     }
   }
   if (hipGetLastError() != hipSuccess) {
