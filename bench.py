@@ -181,6 +181,10 @@ def main():
                          "extension FGMS.backend (plan from its cache); the other one is reported next to it")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run plain 256 MiB device copies (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--pin-weights", type=int, default=-1, choices=[-1, 0, 1],
+                    help="1: promise the library that the weights do not change between calls (fgms_weights_pin: "
+                         "it keeps its re-laid copies), 0: do not; default: 1 for forward-only workloads "
+                         "(inference), 0 for training steps")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (every figure is "
@@ -198,6 +202,11 @@ def main():
     capi.set_kernel_policy(args.policy)
     backend.fgms_set_kernel_policy(args.policy)
     backend.fgms_plan_cache(not args.no_plan)
+
+    pinned = args.pin_weights == 1 or (args.pin_weights < 0 and tuple(passes) == ("fwd",))
+    if pinned:
+        capi.weights_pin(D["kernel"])
+        backend.fgms_weights_pin(D["kernel"])
 
     def make_plan():
         return capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
@@ -466,6 +475,7 @@ def main():
         "config": {"workload": args.workload, "voxels_in": L["n_in"], "voxels_out": L["n_out"],
                    "pairs": m, "k_vol": L["k_vol"], "c_in": L["c_in"], "c_out": L["c_out"],
                    "plan": plan is not None, "policy": args.policy, "surface": args.surface,
+                   "weights_pinned": pinned,
                    "row_slots_per_pair": (round(plan.stats()["blocks_fwd"] * 64.0 / max(plan.stats()["pairs"], 1), 3)
                                           if plan is not None else None)},
         "kernels": kernels,

@@ -18,6 +18,7 @@ SYMBOLS = [
     "fgms_plan_usable", "fgms_plan_stats", "fgms_fusion_fwd", "fgms_fwd", "fgms_bwd", "fgms_dgrad",
     "fgms_wgrad", "fgms_wgrad_static", "fgms_set_kernel_policy", "fgms_profile_enable", "fgms_profile_read",
     "fgms_profile_reset", "fgms_probe_gather", "fgms_build_kernel_map", "fgms_allocation_count",
+    "fgms_weights_pin", "fgms_weights_unpin", "fgms_relaid_weights_hits",
 ]
 
 _lib = None
@@ -67,6 +68,11 @@ def lib():
     L.fgms_set_kernel_policy.argtypes = [i32]
     L.fgms_set_kernel_policy.restype = None
     L.fgms_allocation_count.restype = ctypes.c_longlong
+    L.fgms_relaid_weights_hits.restype = ctypes.c_longlong
+    L.fgms_weights_pin.argtypes = [vp]
+    L.fgms_weights_pin.restype = i32
+    L.fgms_weights_unpin.argtypes = [vp]
+    L.fgms_weights_unpin.restype = i32
     L.fgms_profile_enable.argtypes = [i32]
     L.fgms_profile_enable.restype = None
     L.fgms_profile_reset.restype = None
@@ -120,6 +126,21 @@ def set_kernel_policy(policy):
 def allocation_count():
     """Device / pinned allocations the library has made so far (``fgms_allocation_count``)."""
     return int(lib().fgms_allocation_count())
+
+
+def weights_pin(kernel):
+    """Promise that ``kernel``'s bytes stay as they are until the next pin / unpin of the tensor:
+    the library keeps its re-laid copies (``fgms_weights_pin``).  The caller keeps the tensor alive."""
+    _check(lib().fgms_weights_pin(ctypes.c_void_p(kernel.data_ptr())))
+
+
+def weights_unpin(kernel=None):
+    """Drop the re-laid copies of ``kernel`` (None: of every pinned tensor on the current device)."""
+    _check(lib().fgms_weights_unpin(ctypes.c_void_p(kernel.data_ptr() if kernel is not None else None)))
+
+
+def relaid_weights_hits():
+    return int(lib().fgms_relaid_weights_hits())
 
 
 def profile_enable(on=True):

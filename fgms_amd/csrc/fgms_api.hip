@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <algorithm>
 #include <atomic>
 #include <map>
 #include <mutex>
@@ -91,6 +92,149 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *
   *ptr = b.ptr;
   return FGMS_OK;
 }
+
+// ---- re-laid copies of pinned weights -----------------------------------------
+// Some kernels read the weights from a re-laid copy, made by a small launch in front of the
+// main one (4-9 us where the main launch takes 90).  A caller that promises that a weight
+// tensor's bytes stay as they are (fgms_weights_pin: inference, or between two optimizer
+// steps) lets the library keep those copies, per (address, layout), until fgms_weights_unpin
+// or the next fgms_weights_pin of the address.
+namespace {
+struct RelaidCopy {
+  const void *w;
+  int device;
+  unsigned layout;
+  int k_vol, c_in, c_out;
+  size_t bytes;
+  void *ptr;
+  hipStream_t made_on;
+  hipEvent_t ready;                  // nullptr: the fill has not been queued (yet)
+  std::vector<hipStream_t> users;    // streams other than made_on that wait for `ready` already
+};
+std::mutex g_pin_mutex;
+std::vector<std::pair<int, const void *>> g_pinned;
+std::vector<RelaidCopy> g_relaid;
+std::atomic<int> g_pinned_count{0};
+std::atomic<long long> g_relaid_hits{0};
+
+bool is_pinned_locked(int dev, const void *w) {
+  for (const auto &e : g_pinned)
+    if (e.first == dev && e.second == w) return true;
+  return false;
+}
+
+// Hands a copy's block back to the pool once every stream that read it has passed this point.
+void retire_locked(RelaidCopy &c) {
+  for (hipStream_t s : c.users) {
+    hipEvent_t ev = nullptr;
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) continue;
+    if (hipEventRecord(ev, s) == hipSuccess) (void)hipStreamWaitEvent(c.made_on, ev, 0);
+    (void)hipEventDestroy(ev);
+  }
+  if (c.ready) (void)hipEventDestroy(c.ready);
+  pool_free(c.ptr, c.made_on, false);
+}
+
+void drop_copies_locked(int dev, const void *w) {
+  for (size_t i = 0; i < g_relaid.size();) {
+    if (g_relaid[i].device == dev && g_relaid[i].w == w) {
+      retire_locked(g_relaid[i]);
+      g_relaid.erase(g_relaid.begin() + i);
+    } else {
+      ++i;
+    }
+  }
+}
+}  // namespace
+
+int relaid_weights_buffer(const GmsArgs &a, unsigned layout, size_t bytes, void **ptr, bool *fill) {
+  *fill = true;
+  if (g_pinned_count.load(std::memory_order_relaxed) > 0) {
+    int dev = 0;
+    FGMS_HIP_TRY(hipGetDevice(&dev));
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    const bool capturing = a.stream && hipStreamIsCapturing(a.stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    if (!capturing && is_pinned_locked(dev, a.w)) {
+      for (RelaidCopy &c : g_relaid) {
+        if (c.w != a.w || c.device != dev || c.layout != layout || c.k_vol != a.k_vol || c.c_in != a.c_in ||
+            c.c_out != a.c_out || c.bytes != bytes)
+          continue;
+        *ptr = c.ptr;
+        if (!c.ready) {           // an earlier call failed between the buffer and its fill
+          c.made_on = a.stream;
+          c.users.clear();
+          return FGMS_OK;
+        }
+        if (a.stream != c.made_on && std::find(c.users.begin(), c.users.end(), a.stream) == c.users.end()) {
+          FGMS_HIP_TRY(hipStreamWaitEvent(a.stream, c.ready, 0));
+          c.users.push_back(a.stream);
+        }
+        *fill = false;
+        g_relaid_hits.fetch_add(1, std::memory_order_relaxed);
+        return FGMS_OK;
+      }
+      void *p = nullptr;
+      int rc = pool_alloc(&p, bytes, a.stream);
+      if (rc != FGMS_OK) return rc;
+      g_relaid.push_back(RelaidCopy{a.w, dev, layout, a.k_vol, a.c_in, a.c_out, bytes, p, a.stream, nullptr, {}});
+      *ptr = p;
+      return FGMS_OK;
+    }
+  }
+  return workspace_get(a.stream, 0, bytes, ptr);
+}
+
+void relaid_weights_filled(const GmsArgs &a, void *ptr) {
+  if (g_pinned_count.load(std::memory_order_relaxed) == 0) return;
+  std::lock_guard<std::mutex> lock(g_pin_mutex);
+  for (RelaidCopy &c : g_relaid) {
+    if (c.ptr != ptr || c.ready) continue;
+    hipEvent_t ev = nullptr;
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) return;
+    if (hipEventRecord(ev, a.stream) != hipSuccess) {
+      (void)hipEventDestroy(ev);
+      return;
+    }
+    c.ready = ev;
+    return;
+  }
+}
+
+extern "C" int fgms_weights_pin(const void *kernel) {
+  if (!kernel) {
+    set_error("fgms_weights_pin: null pointer");
+    return FGMS_E_INVALID;
+  }
+  int dev = 0;
+  FGMS_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_pin_mutex);
+  if (is_pinned_locked(dev, kernel)) {
+    drop_copies_locked(dev, kernel);       // pinned again: the bytes have changed since
+  } else {
+    g_pinned.emplace_back(dev, kernel);
+    g_pinned_count.store((int)g_pinned.size(), std::memory_order_relaxed);
+  }
+  return FGMS_OK;
+}
+
+extern "C" int fgms_weights_unpin(const void *kernel) {
+  int dev = 0;
+  FGMS_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_pin_mutex);
+  for (size_t i = 0; i < g_pinned.size();) {
+    if (g_pinned[i].first == dev && (!kernel || g_pinned[i].second == kernel)) {
+      drop_copies_locked(dev, g_pinned[i].second);
+      g_pinned.erase(g_pinned.begin() + i);
+    } else {
+      ++i;
+    }
+  }
+  g_pinned_count.store((int)g_pinned.size(), std::memory_order_relaxed);
+  return FGMS_OK;
+}
+
+extern "C" long long fgms_relaid_weights_hits(void) { return g_relaid_hits.load(std::memory_order_relaxed); }
 
 // ---- dynamic-LDS limits already granted, per (device, kernel) ------------------
 namespace {

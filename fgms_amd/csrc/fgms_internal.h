@@ -187,6 +187,12 @@ struct Plan {
 // all-zero between calls), slot 2: the generic kernel's accumulator, slot 3: the gather probe's sink.
 // *fresh (optional) is set when the buffer was (re)allocated by this call.
 int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *fresh = nullptr);
+// Buffer for a re-laid copy of a.w in `layout` (any number that tells the layouts of one weight
+// tensor apart): the stream's workspace, to be filled (*fill = true), or -- for weights under
+// fgms_weights_pin -- a kept copy that a first call fills (relaid_weights_filled once its fill
+// is queued) and later calls find filled (*fill = false).
+int relaid_weights_buffer(const GmsArgs &a, unsigned layout, size_t bytes, void **ptr, bool *fill);
+void relaid_weights_filled(const GmsArgs &a, void *ptr);
 size_t workspace_bytes(hipStream_t stream, int slot);
 
 // Brackets a main-kernel launch with events when profiling is enabled.

@@ -936,14 +936,34 @@ template <typename T>
 int pack_weights(const GmsArgs &a, const Shape &s, const T **packed) {
   void *ws = nullptr;
   const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
-  int rc = workspace_get(a.stream, 0, n * sizeof(T), &ws);
+  bool fill = true;
+  int rc = relaid_weights_buffer(a, (unsigned)s.S << 8 | (a.transpose_w ? 2u : 0u), n * sizeof(T), &ws, &fill);
   if (rc != FGMS_OK) return rc;
+  *packed = (const T *)ws;
+  if (!fill) return FGMS_OK;
   unsigned blocks = (unsigned)((n + 255) / 256);
   if (blocks > 4096) blocks = 4096;
   pack_weights_kernel<T><<<blocks, 256, 0, a.stream>>>((const T *)a.w, (T *)ws, a.k_vol, a.c_in,
                                                        a.c_out, s.S, a.transpose_w);
   FGMS_HIP_TRY(hipGetLastError());
-  *packed = (const T *)ws;
+  relaid_weights_filled(a, ws);
+  return FGMS_OK;
+}
+
+// The same for the split-bf16 layout of fp32 weights (pack_weights_bf3_kernel).
+int pack_weights_bf3(const GmsArgs &a, bool transpose, const void **packed) {
+  void *ws = nullptr;
+  const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
+  bool fill = true;
+  int rc = relaid_weights_buffer(a, 1u | (transpose ? 2u : 0u), n * sizeof(float), &ws, &fill);
+  if (rc != FGMS_OK) return rc;
+  *packed = ws;
+  if (!fill) return FGMS_OK;
+  size_t blocks = (n / 8 + 255) / 256;
+  pack_weights_bf3_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, a.stream>>>(
+      (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out, transpose);
+  FGMS_HIP_TRY(hipGetLastError());
+  relaid_weights_filled(a, ws);
   return FGMS_OK;
 }
 
@@ -955,14 +975,9 @@ int launch_pairs(const GmsArgs &a, const Shape &s) {
   constexpr bool kCanSplit = sizeof(T) == 4 && S == 4;
   const bool split = kCanSplit && a.reduced && split_bf16_enabled();
   if (split) {
-    void *ws = nullptr;
-    const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
-    int rc = workspace_get(a.stream, 0, n * sizeof(float), &ws);
+    const void *ws = nullptr;
+    int rc = pack_weights_bf3(a, a.transpose_w, &ws);
     if (rc != FGMS_OK) return rc;
-    size_t blocks = (n / 8 + 255) / 256;
-    pack_weights_bf3_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, a.stream>>>(
-        (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out, a.transpose_w);
-    FGMS_HIP_TRY(hipGetLastError());
     packed = (const T *)ws;
   } else {
     int rc = pack_weights<T>(a, s, &packed);
@@ -1075,14 +1090,9 @@ int launch_rows(const GmsArgs &a, const Shape &s, const int32_t *nbr,
   if (kCanSplit && a.reduced && raw == 2 && split_bf16_enabled()) raw = 4;   // (the input gradient splits as it reads)
   const T *packed = raw ? (const T *)a.w : (const T *)a.prepacked;
   if (split) {
-    void *ws = nullptr;
-    const size_t n = (size_t)a.k_vol * a.c_in * a.c_out;
-    int rc = workspace_get(a.stream, 0, n * sizeof(float), &ws);
+    const void *ws = nullptr;
+    int rc = pack_weights_bf3(a, false, &ws);
     if (rc != FGMS_OK) return rc;
-    size_t blocks = (n / 8 + 255) / 256;
-    pack_weights_bf3_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, a.stream>>>(
-        (const float *)a.w, (int4v *)ws, a.k_vol, a.c_in, a.c_out, false);
-    FGMS_HIP_TRY(hipGetLastError());
     packed = (const T *)ws;
     raw = 3;
   } else if (!packed) {

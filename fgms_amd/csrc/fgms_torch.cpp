@@ -14,6 +14,9 @@
 //    queues a fingerprint check of the lists (fgms_plan_check), and the call after
 //    a rewrite raises RuntimeError and drops the plan.  A call with in_map and out_map exchanged (the
 //    transposed convolution over the same pairs) shares the cached plan's tables;
+//  * fgms_weights_pin(kernel) lets the library keep the re-laid copies of a weight tensor that
+//    some kernels read (inference); a forward call that finds the tensor's version counter
+//    moved drops them;
 //  * HIP errors raise RuntimeError instead of passing silently.
 #include <torch/extension.h>
 
@@ -24,6 +27,7 @@
 #include <list>
 #include <mutex>
 #include <stdexcept>
+#include <vector>
 
 #include "fgms.h"
 #include "fgms_diag.h"
@@ -154,6 +158,55 @@ fgms_plan_t *plan_for(const at::Tensor &kpos, const at::Tensor &in_map, const at
   return plan;
 }
 
+// Weight tensors whose re-laid copies the library may keep (fgms_weights_pin): the entry holds
+// the tensor, so that its address cannot go to another tensor meanwhile, and its version counter;
+// a forward call that finds the counter moved pins the address again, which drops the copies.
+struct PinnedWeights {
+  at::Tensor kernel;
+  int64_t version;
+};
+std::vector<PinnedWeights> g_pins;
+
+void pin_weights(const at::Tensor &kernel) {
+  need_contiguous_cuda(kernel, "kernel");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(kernel.device());
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (auto &p : g_pins)
+    if (p.kernel.is_same(kernel)) {
+      p.version = version_of(kernel);
+      check(fgms_weights_pin(kernel.data_ptr()));
+      return;
+    }
+  check(fgms_weights_pin(kernel.data_ptr()));
+  g_pins.push_back(PinnedWeights{kernel, version_of(kernel)});
+}
+
+void unpin_weights(const at::Tensor &kernel) {
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(kernel.device());
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (size_t i = 0; i < g_pins.size(); ++i)
+    if (g_pins[i].kernel.is_same(kernel)) {
+      check(fgms_weights_unpin(kernel.data_ptr()));
+      g_pins.erase(g_pins.begin() + i);
+      return;
+    }
+}
+
+// (with the device guard of the call in place)
+void refresh_pin(const at::Tensor &kernel) {
+  if (g_pins.empty()) return;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (auto &p : g_pins)
+    if (p.kernel.is_same(kernel)) {
+      const int64_t v = version_of(kernel);
+      if (v != p.version) {
+        check(fgms_weights_pin(kernel.data_ptr()));
+        p.version = v;
+      }
+      return;
+    }
+}
+
 void check_channels(const at::Tensor &in_feats, const at::Tensor &kernel) {
   // the reference's one argument check, backend/spconv.cu:39-43
   if (in_feats.size(1) != kernel.size(1))
@@ -174,6 +227,7 @@ void ConvolutionForwardFused(const at::Tensor in_feats, const at::Tensor kernel,
   c10::hip::HIPGuardMasqueradingAsCUDA guard(in_feats.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   const int k_vol = (int)kernel.size(0);
+  refresh_pin(kernel);
   fgms_plan_t *plan = plan_for(kpos, in_map, out_map, in_feats.size(0), out_feats.size(0), k_vol, stream);
   check(fgms_fusion_fwd(in_feats.data_ptr(), kernel.data_ptr(), sum_nnz, out_feats.data_ptr(),
                         i32(kpos), qkpos.defined() && qkpos.numel() ? i32(qkpos) : nullptr,
@@ -198,6 +252,7 @@ void ConvolutionForward(const at::Tensor in_feats, const at::Tensor kernel, cons
   at::Tensor knnz = kernel_nnz.contiguous();
   c10::hip::HIPGuardMasqueradingAsCUDA guard(in_feats.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  refresh_pin(kernel);
   fgms_plan_t *plan = plan_for(kernel_pos, in_map, out_map, in_feats.size(0), out_feats.size(0), k_vol, stream);
   check(fgms_fwd(in_feats.data_ptr(), kernel.data_ptr(), sum_nnz, out_feats.data_ptr(),
                  knnz.data_ptr<int>(), i32(kernel_pos), i32(in_map), i32(out_map), separate_mid,
@@ -238,6 +293,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("fgms_plan_cache_clear", &clear_cache);
   m.def("fgms_plan_cache_size", &cache_size);
   m.def("fgms_plan_cache_views", []() { std::lock_guard<std::mutex> lock(g_mutex); return g_views_made; });
+  m.def("fgms_weights_pin", &pin_weights, pybind11::arg("kernel"));
+  m.def("fgms_weights_unpin", &unpin_weights, pybind11::arg("kernel"));
   m.def("fgms_version", []() { return std::string(fgms_version()); });
   m.def("fgms_set_kernel_policy", &fgms_set_kernel_policy);
 }

@@ -200,6 +200,22 @@ int fgms_wgrad_static(const void *in_feats, const void *out_feats_grad, void *ke
                       int64_t n_pairs, int dtype, fgms_plan_t *plan, void *stream);
 
 /*
+ * Weights that do not change between calls.  No counterpart in the reference, which hands its
+ * kernels the weight tensor as it is (backend/spconv.cu:112-238).  Some kernels here read the
+ * weights from a re-laid copy that a small launch makes in front of the main one (wide fp16
+ * layers, fp32 forward passes: 4-9 us per call).  fgms_weights_pin(kernel) is the caller's
+ * promise that the bytes at `kernel` stay as they are until the next fgms_weights_pin or
+ * fgms_weights_unpin of that address: the library then makes each such copy once and keeps it
+ * (device memory of the tensor's size per layout used, on the current device).  After writing
+ * to the tensor (an optimizer step, loading a checkpoint) call fgms_weights_pin again, which
+ * drops the copies; before freeing it call fgms_weights_unpin (NULL: every pinned address on
+ * the current device).  A call on a pinned tensor whose bytes were changed without this reads
+ * the old weights.  Calls under stream capture and the backward calls do not use the copies.
+ */
+int fgms_weights_pin(const void *kernel);
+int fgms_weights_unpin(const void *kernel);
+
+/*
  * Kernel-map builder.  No counterpart in the reference, whose scripts load the
  * maps from files (cpu-check.py:89-94, spconv-test.py:64-73); this is the step
  * right before the path.  Finds every pair (i, o) with

@@ -60,6 +60,9 @@ int fgms_probe_gather(const void *feats, int c_src, int dtype, int for_dgrad,
 /* How many device or pinned-host allocations (hipMalloc, hipHostMalloc) the library has made
  * since it was loaded: a test can assert that a call made none. */
 long long fgms_allocation_count(void);
+/* How many launches found the re-laid copy of a pinned weight tensor (fgms_weights_pin)
+ * already made, since the library was loaded. */
+long long fgms_relaid_weights_hits(void);
 void fgms_profile_enable(int on);
 int fgms_profile_read(int index, char *name, int name_len, float *ms);
 void fgms_profile_reset(void);

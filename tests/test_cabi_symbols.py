@@ -26,7 +26,7 @@ def test_header_declares_the_reference_entry_points():
         assert s in syms
     # the drop-in header carries no test or measurement entry points
     for s in syms:
-        assert not s.startswith(("fgms_profile", "fgms_probe", "fgms_set_kernel_policy", "fgms_allocation")), s
+        assert not s.startswith(("fgms_profile", "fgms_probe", "fgms_set_kernel_policy", "fgms_allocation", "fgms_relaid")), s
 
 
 def test_library_exports_every_declared_symbol():
