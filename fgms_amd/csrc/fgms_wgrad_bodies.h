@@ -164,6 +164,17 @@ __device__ __forceinline__ void wgrad_wave_body(
   const int nstages = (count + SP - 1) / SP;
   int xi[NX], gi[NG];        // gather rows of the next stage to load
   int4v xr[NX], gr[NG];      // the rows in flight
+  // fp16: a stage's 2 x SP indices arrive through ONE load (lanes 0..SP-1 read the input rows'
+  // indices, lanes 32.. the output rows') and are handed round through 256 bytes of LDS behind
+  // the staging tiles, instead of one load instruction per row instruction: a lane's chunks then
+  // belong to NX (NG) consecutive pairs, whose indices it reads back with one LDS read each.
+  static_assert(!kBufW || (SP == 32 && (NX == 2 || NX == 4) && (NG == 2 || NG == 4)), "index exchange: 32 pairs a stage");
+  int *ibuf = reinterpret_cast<int *>(reinterpret_cast<T *>(lds) + (size_t)4 * SP * (LDI + LDO)) + wave * 64;
+  const int32_t *const my_map = lane < 32 ? imap : omap;
+  int idx_raw = 0;
+  // chunk i of this lane: pair `row`, 16-byte piece `cc` of its row
+  auto x_row = [&](int i) { return kBufW ? (lane / NCI) * NX + i : (lane + 64 * i) / NCI; };
+  auto g_row = [&](int i) { return kBufW ? (lane / NCO) * NG + i : (lane + 64 * i) / NCO; };
 
   // Everything is issued unconditionally and nothing touches a loaded register before
   // its consumer: an index or a row that is selected, copied or loaded under a branch
@@ -171,6 +182,10 @@ __device__ __forceinline__ void wgrad_wave_body(
   // would no longer run under the MFMAs.  Past the end of the slice the last pair is
   // read again; store_rows zeroes those rows by their position instead.
   auto load_idx = [&](int st) {
+    if constexpr (kBufW) {
+      idx_raw = my_map[first + min(st * SP + (lane & 31), count - 1)];
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NX; ++i)
       xi[i] = imap[first + min(st * SP + (lane + 64 * i) / NCI, count - 1)];
@@ -178,12 +193,32 @@ __device__ __forceinline__ void wgrad_wave_body(
     for (int i = 0; i < NG; ++i)
       gi[i] = omap[first + min(st * SP + (lane + 64 * i) / NCO, count - 1)];
   };
+  // fp16: the indices that load_idx fetched last, from idx_raw through LDS into xi / gi
+  auto hand_round = [&]() {
+    ibuf[lane] = idx_raw;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if constexpr (NX == 4) {
+      const int4v v = *reinterpret_cast<const int4v *>(ibuf + (lane / NCI) * 4);
+      xi[0] = v[0]; xi[1] = v[1]; xi[2] = v[2]; xi[3] = v[3];
+    } else {
+      const int2v v = *reinterpret_cast<const int2v *>(ibuf + (lane / NCI) * 2);
+      xi[0] = v[0]; xi[1] = v[1];
+    }
+    if constexpr (NG == 4) {
+      const int4v v = *reinterpret_cast<const int4v *>(ibuf + 32 + (lane / NCO) * 4);
+      gi[0] = v[0]; gi[1] = v[1]; gi[2] = v[2]; gi[3] = v[3];
+    } else {
+      const int2v v = *reinterpret_cast<const int2v *>(ibuf + 32 + (lane / NCO) * 2);
+      gi[0] = v[0]; gi[1] = v[1];
+    }
+  };
   auto load_rows = [&](int st_) {      // st_: the stage the indices in xi / gi belong to
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
-      const int cc = (lane + 64 * i) % NCI;
+      const int cc = kBufW ? lane % NCI : (lane + 64 * i) % NCI;
       if constexpr (kBufW) {
-        const bool live = st_ * SP + (lane + 64 * i) / NCI < count;
+        const bool live = st_ * SP + x_row(i) < count;
         const unsigned off = live ? (unsigned)xi[i] * (unsigned)(c_in * (int)sizeof(T)) : kAbsentRow;
         xr[i] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(
                                               in_rsrc, off + (unsigned)((ci0 + cc * E) * (int)sizeof(T)), 0, 0));
@@ -193,9 +228,9 @@ __device__ __forceinline__ void wgrad_wave_body(
     }
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-      const int cc = (lane + 64 * i) % NCO;
+      const int cc = kBufW ? lane % NCO : (lane + 64 * i) % NCO;
       if constexpr (kBufW) {
-        const bool live = st_ * SP + (lane + 64 * i) / NCO < count;
+        const bool live = st_ * SP + g_row(i) < count;
         const unsigned off = live ? (unsigned)gi[i] * (unsigned)(c_out * (int)sizeof(T)) : kAbsentRow;
         gr[i] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(
                                               gout_rsrc, off + (unsigned)((co0 + cc * E) * (int)sizeof(T)), 0, 0));
@@ -211,7 +246,7 @@ __device__ __forceinline__ void wgrad_wave_body(
       if constexpr (SPLIT)
         store_split_chunk(xh, xl, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count, lane);
       else if constexpr (kBufW)
-        *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) = xr[i];
+        *reinterpret_cast<int4v *>(x + x_row(i) * LDI + (lane % NCI) * E) = xr[i];
       else
         *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
             st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
@@ -222,7 +257,7 @@ __device__ __forceinline__ void wgrad_wave_body(
       if constexpr (SPLIT)
         store_split_chunk(gh, gl, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count, lane);
       else if constexpr (kBufW)
-        *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) = gr[i];
+        *reinterpret_cast<int4v *>(g + g_row(i) * LDO + (lane % NCO) * E) = gr[i];
       else
         *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
             st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
@@ -235,11 +270,13 @@ __device__ __forceinline__ void wgrad_wave_body(
 
   int st = wave;
   load_idx(st);
+  if constexpr (kBufW) hand_round();
   load_rows(st);
   load_idx(st + 4);
   while (st < nstages) {
     store_rows(st);                 // waits for the stage's rows
-    wave_fence();
+    if constexpr (kBufW) hand_round();   // (the indices of stage st + 4 came in behind them)
+    else wave_fence();
     load_rows(st + 4);              // stage st + 4, in flight during the MFMAs
     __builtin_amdgcn_sched_barrier(0);   // (rows first, then indices, both before the MFMAs:
     load_idx(st + 8);                    //  the wait for the rows then leaves the indices in flight)
