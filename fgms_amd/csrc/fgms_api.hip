@@ -147,6 +147,14 @@ void drop_copies_locked(int dev, const void *w) {
 }
 }  // namespace
 
+bool weights_pinned(const void *w) {
+  if (g_pinned_count.load(std::memory_order_relaxed) == 0) return false;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  std::lock_guard<std::mutex> lock(g_pin_mutex);
+  return is_pinned_locked(dev, w);
+}
+
 int relaid_weights_buffer(const GmsArgs &a, unsigned layout, size_t bytes, void **ptr, bool *fill) {
   *fill = true;
   if (g_pinned_count.load(std::memory_order_relaxed) > 0) {

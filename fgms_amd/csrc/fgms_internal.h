@@ -193,6 +193,7 @@ int workspace_get(hipStream_t stream, int slot, size_t bytes, void **ptr, bool *
 // is queued) and later calls find filled (*fill = false).
 int relaid_weights_buffer(const GmsArgs &a, unsigned layout, size_t bytes, void **ptr, bool *fill);
 void relaid_weights_filled(const GmsArgs &a, void *ptr);
+bool weights_pinned(const void *w);   // under fgms_weights_pin on the current device
 size_t workspace_bytes(hipStream_t stream, int slot);
 
 // Brackets a main-kernel launch with events when profiling is enabled.

@@ -80,19 +80,25 @@ def test_pinned_copy_is_made_once_and_changes_nothing(capi, oracle, dtype, c_in,
     capi.set_kernel_policy(0)
 
 
-def test_backward_and_raw_weight_kernels_ignore_the_pin(capi, oracle):
-    """64 -> 64 fp16 reads the weight tensor as it is: pinning it makes no copy and no hit."""
+def test_pinned_fp16_forward_reads_the_copy_and_the_backward_call_does_not(capi, oracle):
+    """64 -> 64 fp16 reads the weight tensor as it lies; pinned, the forward pass takes the kept
+    re-laid copy instead (plain instead of transposing fragment reads), the backward call still
+    reads the tensor itself."""
     L = layer(np.float16, 64, 64)
     D = G.to_dev(L)
     plan = capi.Plan(D["kpos"], D["imap"], D["omap"], D["n_in"], D["n_out"])
+    a = (L["knnz"], L["imap"], L["omap"])
+    raw = G.run_fwd(capi, D, plan=plan)
     capi.weights_pin(D["kernel"])
     h0 = capi.relaid_weights_hits()
     out = G.run_fwd(capi, D, plan=plan)
     out2 = G.run_fwd(capi, D, plan=plan)
+    assert capi.relaid_weights_hits() == h0 + 1
     gi, gw = G.run_bwd(capi, D, plan=plan)
-    assert capi.relaid_weights_hits() == h0
-    a = (L["knnz"], L["imap"], L["omap"])
-    G.assert_close(out, oracle.c_fwd(L["in_feats"], L["kernel"], *a, L["n_out"]), "fp16", "fwd")
+    assert capi.relaid_weights_hits() == h0 + 1
+    ref = oracle.c_fwd(L["in_feats"], L["kernel"], *a, L["n_out"])
+    G.assert_close(raw, ref, "fp16", "fwd, weights as they lie")
+    G.assert_close(out, ref, "fp16", "fwd, pinned")
     assert np.array_equal(out, out2)
     G.assert_close(gi, oracle.c_dgrad(L["out_grad"], L["kernel"], *a, L["n_in"]), "fp16", "dgrad")
     capi.weights_unpin(D["kernel"])
