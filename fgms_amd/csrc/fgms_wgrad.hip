@@ -402,7 +402,7 @@ int wgrad_geometry(const WgradArgs &a, WgradGeometry *g, bool shares_grid) {
     // fp32 tensors whose caller allows tf32 precision: four 16-bit tiles per wave instead
     g->split = !f16 && a.reduced && split_bf16_enabled();
     const size_t lds = (g->split ? 4 * (size_t)sp * 2 * ((bi * 32 + 16) + (bj * 32 + 16)) * 2
-                                 : 4 * (size_t)sp * ((bi * 32 + pad) + (bj * 32 + pad)) * esz)
+                                 : 4 * (size_t)sp * ((bi * 32 + (f16 ? 0 : pad)) + (bj * 32 + (f16 ? 0 : pad))) * esz)
                        + 4 * 64 * sizeof(int);                           // + the waves' index exchange
     const size_t red = 3 * (size_t)bi * bj * 16 * 64 * sizeof(float);     // the partial tiles' exchange
     g->lds = lds < red ? red : lds;

@@ -38,6 +38,23 @@ __device__ __forceinline__ half8 tr_frag(const __half *tile, int ld, int p0, int
   return __builtin_bit_cast(half8, v);
 }
 
+// The same from a tile without row padding (rows of exactly `ld` = 32 or 64 halfs).  One
+// transposing read touches rows p .. p + 3 and p + 8 .. p + 11, 64 bytes of each; with 128-byte
+// rows, rows p and p + 2 would meet in the same banks, so the writer exchanges the two 64-byte
+// halves of every row whose (row >> 1) is odd (wave tile below) and the read does the same.
+template <int LD>
+__device__ __forceinline__ half8 tr_frag_dense(const __half *tile, int p0, int c0, int lane) {
+  static_assert(LD == 32 || LD == 64, "dense tile: 32 or 64 channels a row");
+  const int b = lane >> 4, i = lane & 15, h = lane >> 5;
+  const int sw = LD == 64 ? ((lane >> 3) & 1) * 32 : 0;
+  const __half *base = tile + (size_t)(p0 + h * 8 + (i >> 2)) * LD + (c0 ^ sw) + (b & 1) * 16 + (i & 3) * 4;
+  typedef __attribute__((address_space(3))) short4v lds_v4;
+  const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4 *)(base));
+  const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4 *)(base + 4 * LD));
+  const short8v v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(half8, v);
+}
+
 // Workgroup -> (slice sl of the pair list, offset k) and the slice's pair range.
 // Workgroups go to the 8 XCDs round-robin; numbering them so that one XCD gets
 // all the offsets of a slice lets the rows one offset pulled into that XCD's L2
@@ -134,7 +151,8 @@ __device__ __forceinline__ void wgrad_wave_body(
   constexpr bool kBufW = sizeof(T) == 2 && !SPLIT;
   const __amdgpu_buffer_rsrc_t in_rsrc = rows_resource(in, in_bytes), gout_rsrc = rows_resource(gout, gout_bytes);
   constexpr int CI = BI * 32, CO = BJ * 32;
-  constexpr int LDI = CI + W::pad, LDO = CO + W::pad;
+  // (fp16: rows without padding, 64-byte halves exchanged by row instead, see tr_frag_dense)
+  constexpr int LDI = CI + (kBufW ? 0 : W::pad), LDO = CO + (kBufW ? 0 : W::pad);
   constexpr int NCI = CI / E, NCO = CO / E;
   constexpr int NX = SP * NCI / 64, NG = SP * NCO / 64;   // chunks per lane and stage
   static_assert(NX >= 1 && NG >= 1, "stage too small");
@@ -246,7 +264,7 @@ __device__ __forceinline__ void wgrad_wave_body(
       if constexpr (SPLIT)
         store_split_chunk(xh, xl, LDIh, e / NCI, e % NCI, xr[i], st * SP + e / NCI < count, lane);
       else if constexpr (kBufW)
-        *reinterpret_cast<int4v *>(x + x_row(i) * LDI + (lane % NCI) * E) = xr[i];
+        *reinterpret_cast<int4v *>(x + x_row(i) * LDI + (((lane % NCI) ^ (CI == 64 ? ((x_row(i) >> 1) & 1) * 4 : 0)) * E)) = xr[i];
       else
         *reinterpret_cast<int4v *>(x + (e / NCI) * LDI + (e % NCI) * E) =
             st * SP + e / NCI < count ? xr[i] : int4v{0, 0, 0, 0};
@@ -257,7 +275,7 @@ __device__ __forceinline__ void wgrad_wave_body(
       if constexpr (SPLIT)
         store_split_chunk(gh, gl, LDOh, e / NCO, e % NCO, gr[i], st * SP + e / NCO < count, lane);
       else if constexpr (kBufW)
-        *reinterpret_cast<int4v *>(g + g_row(i) * LDO + (lane % NCO) * E) = gr[i];
+        *reinterpret_cast<int4v *>(g + g_row(i) * LDO + (((lane % NCO) ^ (CO == 64 ? ((g_row(i) >> 1) & 1) * 4 : 0)) * E)) = gr[i];
       else
         *reinterpret_cast<int4v *>(g + (e / NCO) * LDO + (e % NCO) * E) =
             st * SP + e / NCO < count ? gr[i] : int4v{0, 0, 0, 0};
@@ -307,9 +325,9 @@ __device__ __forceinline__ void wgrad_wave_body(
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-        for (int ti = 0; ti < BI; ++ti) a[ks][ti] = tr_frag(x, LDI, ks * KP, ti * 32, lane);
+        for (int ti = 0; ti < BI; ++ti) a[ks][ti] = tr_frag_dense<CI>(x, ks * KP, ti * 32, lane);
 #pragma unroll
-        for (int tj = 0; tj < BJ; ++tj) b[ks][tj] = tr_frag(g, LDO, ks * KP, tj * 32, lane);
+        for (int tj = 0; tj < BJ; ++tj) b[ks][tj] = tr_frag_dense<CO>(g, ks * KP, tj * 32, lane);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
