@@ -1,6 +1,6 @@
 """The library reads a few switches from the environment once per process (they exist for
 comparisons and experiments).  Each alternative path still has to give the right answer:
-a child process per setting runs forward and backward of two layers through the C ABI,
+a child process per setting runs forward and backward of four layers through the C ABI,
 checks them against the CPU oracle and reports which kernels ran."""
 import json
 import os
@@ -22,7 +22,7 @@ from oracle import fgms_oracle as oracle
 from tests import gpu_util as G
 from tests.test_gpu_parity import layer
 names = set()
-for shape, dtype in (((64, 64), np.float16), ((128, 128), np.float16), ((32, 64), np.float32)):
+for shape, dtype in (((64, 64), np.float16), ((128, 128), np.float16), ((64, 128), np.float16), ((32, 64), np.float32)):
     L = layer(41, shape[0], shape[1], dtype)
     D = G.to_dev(L)
     capi.set_kernel_policy(4)
